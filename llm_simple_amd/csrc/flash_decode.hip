@@ -1,0 +1,340 @@
+// GQA-aware split-KV decode attention for gfx950 (MI355X).
+//
+// The reference decodes with the same operator as prefill, m = 1 and offset =
+// n - 1 (npu_flash_attn_gqa_layer, src/llama2_layer_npu.cpp:866-869): one
+// softmax row per head over the whole contiguous KV cache
+// [max_seq_len][Hkv][128] (src/llama2_layer_npu.cpp:1148-1149).  That is a
+// pure stream of K and V through the chip, so the kernel is organised around
+// HBM: grid = (KV split, kv head, sequence); each workgroup owns a contiguous
+// run of keys of one kv head, each of its 4 waves takes 32 keys per step, and
+// K and V of every key are read from HBM exactly once for all group_size query
+// heads (and all m <= 16/group_size query rows) that share the kv head.
+//
+// The m*group_size query rows are the 16 columns of mfma_f32_16x16x32
+// (S^T = K Q^T, O^T += V^T P^T); unused columns are zero.  K fragments go from
+// global memory straight into the A-operand layout (64 contiguous bytes per
+// 4 lanes); V is staged in a wave-private LDS region and read transposed with
+// ds_read_b64_tr_b16.  Each wave keeps its own running (max, sum, O); the four
+// waves are merged through LDS at the end and the workgroup writes either the
+// final rows (one split) or an fp32 partial (max, sum, unnormalised O) that
+// flash_decode_combine_kernel folds with the log-sum-exp rule.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace llmhip {
+
+constexpr int kDecThreads = 256;
+constexpr int kDecWaveKeys = 32;                  // keys per wave per step
+constexpr int kDecStepKeys = 4 * kDecWaveKeys;    // keys per workgroup per step
+constexpr int kDecCols = 16;                      // query rows per kv head (MFMA N)
+constexpr int kDecWaveLds = kDecWaveKeys * kRowBytes;  // 8 KiB V staging per wave
+
+struct DecodeParams {
+  const char *q;
+  const char *k;
+  const char *v;
+  char *out;
+  float *ws_o;   // [batch][Hkv][splits][16][128]
+  float *ws_ml;  // [batch][Hkv][splits][16][2]
+  int batch, m, n, offset;
+  int64_t kv_seq_stride;
+  int g, Hkv, H;
+  int rows;  // m * g
+  int num_splits, chunk;
+  float scale_log2e;
+};
+
+// V staging swizzle for the 16x16x32 transposed reads: one instruction touches
+// 8 rows x 32 bytes per half-wave, so the 32-byte slot index is XORed with
+// row%8.
+__device__ __forceinline__ int v_swizzle32_off(int row, int granule) {
+  return row * kRowBytes + ((((granule >> 1) ^ (row & 7)) << 5) | ((granule & 1) << 4));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams p) {
+  using E = Elem<T>;
+  __shared__ __attribute__((aligned(16))) char lds[4 * kDecWaveLds + 4 * kDecCols * 2 * 4];
+
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int col = lane & 15, cg = lane >> 4;
+
+  const int k_begin = split * p.chunk;
+  const int k_end = min(p.n, k_begin + p.chunk);
+  const int span = max(k_end - k_begin, 0);
+  const int iters = (span + kDecStepKeys - 1) / kDecStepKeys;
+
+  const size_t kv_row_bytes = (size_t)p.Hkv * kRowBytes;
+  const size_t seq_off = (size_t)b * p.kv_seq_stride * kv_row_bytes + (size_t)kvh * kRowBytes;
+  const char *kbase = p.k + seq_off;
+  const char *vbase = p.v + seq_off;
+
+  // query column of this lane
+  const bool col_valid = col < p.rows;
+  const int c_row = col_valid ? col / p.g : 0;
+  const int c_head = kvh * p.g + (col_valid ? col % p.g : 0);
+  const int c_limit = c_row + p.offset;  // last visible key of this column
+
+  u32x4_t qf[4];
+  {
+    const char *qp = p.q + (((size_t)b * p.m + c_row) * p.H + c_head) * kRowBytes + cg * 16;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      u32x4_t z = {0u, 0u, 0u, 0u};
+      qf[kk] = col_valid ? global_load_b128(qp + kk * 64) : z;
+    }
+  }
+
+  f32x4_t o[8];
+#pragma unroll
+  for (int d = 0; d < 8; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  char *vl = lds + wave * kDecWaveLds;
+
+  u32x4_t kn[2][4], vn[8];
+  auto issue_loads = [&](int it) {
+    const int kb0 = k_begin + it * kDecStepKeys + wave * kDecWaveKeys;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      const int key = min(kb0 + blk * 16 + col, p.n - 1);
+      const char *kp = kbase + (size_t)key * kv_row_bytes + cg * 16;
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) kn[blk][kk] = global_load_b128(kp + kk * 64);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int key = min(kb0 + 4 * i + cg, p.n - 1);
+      vn[i] = global_load_b128(vbase + (size_t)key * kv_row_bytes + col * 16);
+    }
+  };
+
+  if (iters > 0) issue_loads(0);
+
+  for (int it = 0; it < iters; ++it) {
+    const int kb0 = k_begin + it * kDecStepKeys + wave * kDecWaveKeys;
+    u32x4_t kc[2][4];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) kc[blk][kk] = kn[blk][kk];
+    // stage V (rows 4i+cg, granule col) in this wave's LDS region
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lds_write_b128(vl, v_swizzle32_off(4 * i + cg, col), vn[i]);
+    __builtin_amdgcn_wave_barrier();
+    if (it + 1 < iters) issue_loads(it + 1);
+
+    if (kb0 < k_end) {
+      // ---- S^T = K Q^T : 2 blocks of 16 keys ----
+      f32x4_t s[2];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        s[blk] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) s[blk] = E::mfma16(kc[blk][kk], qf[kk], s[blk]);
+      }
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb0 + blk * 16 + 4 * cg + i;
+          float t = s[blk][i] * p.scale_log2e;
+          if (key >= k_end || key > c_limit) t = -INFINITY;
+          s[blk][i] = t;
+          mloc = fmaxf(mloc, t);
+        }
+      mloc = fmaxf(mloc, xor_lane(mloc, 16));
+      mloc = fmaxf(mloc, xor_lane(mloc, 32));
+      const float m_new = fmaxf(m_run, mloc);
+      const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float alpha = fast_exp2(m_run - m_use);
+      m_run = m_new;
+      float psum = 0.0f;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float e = fast_exp2(s[blk][i] - m_use);
+          s[blk][i] = e;
+          psum += e;
+        }
+      l_run = l_run * alpha + psum;
+      // P^T as B operand: slot e<4 -> block 0 key 4cg+e, e>=4 -> block 1 key 4cg+e-4
+      u32x4_t pf;
+      pf[0] = E::pack2(s[0][0], s[0][1]);
+      pf[1] = E::pack2(s[0][2], s[0][3]);
+      pf[2] = E::pack2(s[1][0], s[1][1]);
+      pf[3] = E::pack2(s[1][2], s[1][3]);
+      // ---- O^T += V^T P^T ----
+      const int vr = 4 * cg + (col >> 2);
+      const int sub = (col & 1) * 8;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        const int gran = 2 * d + ((col & 3) >> 1);
+        const u32x2_t lo = lds_read_tr16(vl, v_swizzle32_off(vr, gran) + sub);
+        const u32x2_t hi = lds_read_tr16(vl, v_swizzle32_off(vr + 16, gran) + sub);
+        const u32x4_t vf = {lo[0], lo[1], hi[0], hi[1]};
+        f32x4_t acc = o[d];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] *= alpha;
+        o[d] = E::mfma16(vf, pf, acc);
+      }
+    }
+  }
+
+  // ---- merge the four waves ----
+  float l_tot = l_run + xor_lane(l_run, 16);
+  l_tot += xor_lane(l_tot, 32);
+  __syncthreads();
+  float *lo_f = reinterpret_cast<float *>(lds);                      // [wave][col][128]
+  float *lml = reinterpret_cast<float *>(lds + 4 * kDecWaveLds);     // [wave][col][2]
+#pragma unroll
+  for (int d = 0; d < 8; ++d)
+    *reinterpret_cast<f32x4_t *>(lo_f + ((wave * kDecCols + col) * kHeadDim + 16 * d + 4 * cg)) = o[d];
+  if (cg == 0) {
+    lml[(wave * kDecCols + col) * 2] = m_run;
+    lml[(wave * kDecCols + col) * 2 + 1] = l_tot;
+  }
+  __syncthreads();
+
+  {
+    const int c = tid >> 4, dch = tid & 15;  // column, 8-wide d chunk
+    float mw[4], M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      mw[w] = lml[(w * kDecCols + c) * 2];
+      M = fmaxf(M, mw[w]);
+    }
+    const float M_use = (M == -INFINITY) ? 0.0f : M;
+    float L = 0.0f, acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float wt = fast_exp2(mw[w] - M_use);
+      L += wt * lml[(w * kDecCols + c) * 2 + 1];
+      const float *src = lo_f + ((w * kDecCols + c) * kHeadDim + 8 * dch);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] += wt * src[j];
+    }
+    if (c < p.rows) {
+      if (p.num_splits == 1) {
+        const float inv = (L > 0.0f) ? 1.0f / L : 0.0f;
+        const int r = c / p.g, hq = c % p.g;
+        char *op = p.out + (((size_t)b * p.m + r) * p.H + kvh * p.g + hq) * kRowBytes + dch * 16;
+        u32x4_t w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = E::pack2(acc[2 * j] * inv, acc[2 * j + 1] * inv);
+        *reinterpret_cast<u32x4_t *>(op) = w;
+      } else {
+        const size_t slot = (((size_t)b * p.Hkv + kvh) * p.num_splits + split) * kDecCols + c;
+        float *wo = p.ws_o + slot * kHeadDim + 8 * dch;
+        *reinterpret_cast<f32x4_t *>(wo) = f32x4_t{acc[0], acc[1], acc[2], acc[3]};
+        *reinterpret_cast<f32x4_t *>(wo + 4) = f32x4_t{acc[4], acc[5], acc[6], acc[7]};
+        if (dch == 0) {
+          p.ws_ml[slot * 2] = M;
+          p.ws_ml[slot * 2 + 1] = L;
+        }
+      }
+    }
+  }
+}
+
+// grid (rows, Hkv, batch), 128 threads: thread d folds the splits of one
+// output row with the log-sum-exp rule.
+template <typename T>
+__global__ __launch_bounds__(128) void flash_decode_combine_kernel(DecodeParams p) {
+  using E = Elem<T>;
+  const int c = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int d = threadIdx.x;
+  const size_t base = ((size_t)b * p.Hkv + kvh) * p.num_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < p.num_splits; ++s) M = fmaxf(M, p.ws_ml[((base + s) * kDecCols + c) * 2]);
+  const float M_use = (M == -INFINITY) ? 0.0f : M;
+  float L = 0.0f, acc = 0.0f;
+  for (int s = 0; s < p.num_splits; ++s) {
+    const size_t slot = (base + s) * kDecCols + c;
+    const float wt = fast_exp2(p.ws_ml[slot * 2] - M_use);
+    L += wt * p.ws_ml[slot * 2 + 1];
+    acc += wt * p.ws_o[slot * kHeadDim + d];
+  }
+  const float inv = (L > 0.0f) ? 1.0f / L : 0.0f;
+  const int r = c / p.g, hq = c % p.g;
+  uint16_t *op = reinterpret_cast<uint16_t *>(
+      p.out + (((size_t)b * p.m + r) * p.H + kvh * p.g + hq) * kRowBytes);
+  op[d] = E::round(acc * inv);
+}
+
+static int decode_chunk(int n, int num_splits) {
+  int chunk = (n + num_splits - 1) / num_splits;
+  chunk = ((chunk + kDecStepKeys - 1) / kDecStepKeys) * kDecStepKeys;
+  return chunk;
+}
+
+int flash_decode_default_splits(int batch, int n, int kv_head_num) {
+  // enough workgroups to put ~4 on every one of the 256 CUs, but at least two
+  // steps (256 keys) of work in each split
+  const long long pairs = (long long)batch * kv_head_num;
+  long long want = (1024 + pairs - 1) / pairs;
+  long long cap = n / (2 * kDecStepKeys);
+  if (cap < 1) cap = 1;
+  if (want > cap) want = cap;
+  if (want < 1) want = 1;
+  if (want > 256) want = 256;
+  // drop splits that rounding the chunk up to whole steps would leave empty
+  const int chunk = decode_chunk(n, (int)want);
+  return (n + chunk - 1) / chunk;
+}
+
+size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,
+                                    int num_splits) {
+  (void)m;
+  (void)group_size;
+  if (num_splits <= 1) return 0;
+  const size_t slots = (size_t)batch * kv_head_num * num_splits * kDecCols;
+  return slots * (kHeadDim + 2) * sizeof(float);
+}
+
+hipError_t launch_flash_decode(void *out, const void *q, const void *k, const void *v,
+                               void *workspace, int batch, int m, int n, int offset,
+                               int64_t kv_seq_stride, int group_size, int kv_head_num,
+                               int num_splits, int dt, hipStream_t stream) {
+  DecodeParams p;
+  p.q = static_cast<const char *>(q);
+  p.k = static_cast<const char *>(k);
+  p.v = static_cast<const char *>(v);
+  p.out = static_cast<char *>(out);
+  p.batch = batch;
+  p.m = m;
+  p.n = n;
+  p.offset = offset;
+  p.kv_seq_stride = kv_seq_stride;
+  p.g = group_size;
+  p.Hkv = kv_head_num;
+  p.H = group_size * kv_head_num;
+  p.rows = m * group_size;
+  p.chunk = decode_chunk(n, num_splits);
+  p.num_splits = (n + p.chunk - 1) / p.chunk;  // never more than asked for
+  p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
+  const size_t slots = (size_t)batch * kv_head_num * p.num_splits * kDecCols;
+  p.ws_o = static_cast<float *>(workspace);
+  p.ws_ml = p.ws_o ? p.ws_o + slots * kHeadDim : nullptr;
+  dim3 grid(p.num_splits, kv_head_num, batch);
+  if (dt == kDtFloat16)
+    hipLaunchKernelGGL(flash_decode_kernel<_Float16>, grid, dim3(kDecThreads), 0, stream, p);
+  else
+    hipLaunchKernelGGL(flash_decode_kernel<__bf16>, grid, dim3(kDecThreads), 0, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || p.num_splits == 1) return e;
+  dim3 cgrid(p.rows, kv_head_num, batch);
+  if (dt == kDtFloat16)
+    hipLaunchKernelGGL(flash_decode_combine_kernel<_Float16>, cgrid, dim3(128), 0, stream, p);
+  else
+    hipLaunchKernelGGL(flash_decode_combine_kernel<__bf16>, cgrid, dim3(128), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace llmhip

@@ -1,0 +1,30 @@
+// Launchers of the gfx950 kernels; called only by the C ABI in llmhip.hip after
+// it has validated every argument.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace llmhip {
+
+hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
+                                int n, int offset, int group_size, int kv_head_num, int dt,
+                                hipStream_t stream);
+
+// Split-KV decode.  rows = m * group_size <= 16 query rows per kv head.
+size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,
+                                    int num_splits);
+int flash_decode_default_splits(int batch, int n, int kv_head_num);
+hipError_t launch_flash_decode(void *out, const void *q, const void *k, const void *v,
+                               void *workspace, int batch, int m, int n, int offset,
+                               int64_t kv_seq_stride, int group_size, int kv_head_num,
+                               int num_splits, int dt, hipStream_t stream);
+
+// q_heads may be 0 (rotate K only) and cache pointers may be null (no append):
+// covers rope, rope_single and the fused rope + KV append.
+hipError_t launch_rope_kv_append(void *out_q, void *out_k, void *out_v, const void *freq_cis,
+                                 const void *in_q, const void *in_k, const void *in_v,
+                                 int start_pos, int cur_size, int q_heads, int k_heads,
+                                 int k_out_row_offset, int is_neox, int dt, hipStream_t stream);
+
+}  // namespace llmhip

@@ -1,0 +1,64 @@
+"""Shared helpers of the parity tests: seeded inputs rounded once to the storage
+type and fed, bit for bit, to both the oracle and the HIP path (the reference's
+round-trip trick, tests/flash_attn_test.cpp:88-104)."""
+import numpy as np
+
+from oracle import oracle as orc
+
+DT_FLOAT16 = 4
+DT_BFLOAT16 = 5
+TOL = {DT_FLOAT16: 2e-3, DT_BFLOAT16: 1e-2}  # max-abs bound on the normalised P.V output
+DT_NAME = {DT_FLOAT16: "fp16", DT_BFLOAT16: "bf16"}
+
+
+def normal_bits(seed, shape, dt, scale=1.0):
+    """N(0, scale^2) from the seed, rounded to the storage type: uint16 bits."""
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal(shape, dtype=np.float32) * np.float32(scale)).astype(np.float32)
+    return orc.round_to(x, dt)
+
+
+def to_dev(bits):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).cuda()
+
+
+def dev_empty(shape):
+    import torch
+    return torch.empty(shape, dtype=torch.int16, device="cuda")
+
+
+def to_host(t):
+    return t.cpu().numpy().view(np.uint16)
+
+
+def f32_dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def ulp(x, dt):
+    """Spacing of the storage type at |x| (normal range)."""
+    mant = 7 if dt == DT_BFLOAT16 else 10
+    ax = np.maximum(np.abs(np.asarray(x, dtype=np.float64)), 2.0 ** -14)
+    return 2.0 ** (np.floor(np.log2(ax)) - mant)
+
+
+def check_attention(out_bits, q, k, v, n, offset, dt, batch=None):
+    """Compare HIP output bits with both oracles.
+
+    Against the fp32 oracle (the reference's test golden): max-abs <= TOL, the
+    bar BASELINE sets.  Against the layer-style oracle, whose output is itself
+    rounded to the storage type: within TOL, or on the adjacent representable
+    value (two roundings of nearby reals can land one step apart, and one bf16
+    step at |x| >= 2 is already 1.6e-2)."""
+    got = orc.widen(out_bits, dt)
+    ref32 = orc.attention_f32(q, k, v, n, offset, dt, batch=batch)
+    ref16 = orc.widen(orc.attention_layer(q, k, v, n, offset, dt, batch=batch), dt)
+    assert np.isfinite(got).all()
+    e32 = float(np.abs(got - ref32).max())
+    assert e32 <= TOL[dt], f"max-abs vs fp32 oracle {e32} > {TOL[dt]}"
+    d16 = np.abs(got - ref16)
+    ok = (d16 <= TOL[dt]) | (d16 <= ulp(ref16, dt) * 1.0001)
+    assert ok.all(), f"{np.count_nonzero(~ok)} elements off the layer-style oracle, worst {d16.max()}"
+    return e32, float(d16.max())

@@ -1,0 +1,186 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle
+on identical seeded inputs.  Bit-exact for RoPE and the KV append; max-abs
+<= 2e-3 (fp16) / 1e-2 (bf16) on the attention output."""
+import numpy as np
+import pytest
+
+from helpers import (DT_BFLOAT16, DT_FLOAT16, DT_NAME, TOL, check_attention, dev_empty, f32_dev,
+                     normal_bits, to_dev, to_host)
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    import llm_simple_amd.ops as ops
+    return ops
+
+
+# ---------------------------------------------------------------- RoPE
+
+@pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
+@pytest.mark.parametrize("is_neox", [False, True])
+@pytest.mark.parametrize("cur_size,start_pos,n_heads", [(1, 0, 1), (1, 511, 32), (7, 3, 12), (256, 0, 28), (33, 2015, 4)])
+def test_rope_single_bit_exact(dt, is_neox, cur_size, start_pos, n_heads):
+    ops = _ops()
+    theta = 10000.0 if dt == DT_FLOAT16 else 1e6
+    table = orc.init_freq_cis(128, 2048, theta, dt)
+    x = normal_bits(100 + cur_size + n_heads, (cur_size, n_heads, 128), dt)
+    want = orc.rope(x, table, start_pos, is_neox, dt)
+    d_out = dev_empty(x.shape)
+    ops.hip_rope_single_layer(d_out, f32_dev(table), to_dev(x), start_pos, cur_size, n_heads,
+                              n_heads * 128, is_neox, dt)
+    got = to_host(d_out)
+    assert np.array_equal(got, want), f"{np.count_nonzero(got != want)} elements differ"
+
+
+@pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
+@pytest.mark.parametrize("is_neox", [False, True])
+def test_rope_pair_bit_exact(dt, is_neox):
+    ops = _ops()
+    table = orc.init_freq_cis(128, 1024, 10000.0, dt)
+    q = normal_bits(7, (19, 8, 128), dt)
+    k = normal_bits(8, (19, 8, 128), dt)
+    d_q, d_k = dev_empty(q.shape), dev_empty(k.shape)
+    ops.hip_rope_layer(d_q, d_k, f32_dev(table), to_dev(q), to_dev(k), 100, 19, 8, 8 * 128,
+                       is_neox, dt)
+    assert np.array_equal(to_host(d_q), orc.rope(q, table, 100, is_neox, dt))
+    assert np.array_equal(to_host(d_k), orc.rope(k, table, 100, is_neox, dt))
+
+
+@pytest.mark.parametrize("dt,H,Hkv,theta", [(DT_FLOAT16, 32, 32, 1e4), (DT_BFLOAT16, 12, 2, 1e6), (DT_BFLOAT16, 28, 4, 1e6)])
+@pytest.mark.parametrize("is_neox", [False, True])
+@pytest.mark.parametrize("cur_size,start_pos", [(1, 511), (256, 0), (5, 250)])
+def test_rope_kv_append_bit_exact(dt, H, Hkv, theta, is_neox, cur_size, start_pos):
+    """Fused launch == unfused rope -> copy sequence of the oracle; rows outside
+    [start_pos, start_pos+cur_size) of both caches keep their canary bytes."""
+    ops = _ops()
+    max_seq = 512
+    table = orc.init_freq_cis(128, max_seq, theta, dt)
+    q = normal_bits(1, (cur_size, H, 128), dt)
+    k = normal_bits(2, (cur_size, Hkv, 128), dt)
+    v = normal_bits(3, (cur_size, Hkv, 128), dt)
+    canary_k = np.full((max_seq, Hkv, 128), 0xBEEF, dtype=np.uint16)
+    canary_v = np.full((max_seq, Hkv, 128), 0xCAFE, dtype=np.uint16)
+    want_k, want_v = canary_k.copy(), canary_v.copy()
+    orc.kv_append(want_k, orc.rope(k, table, start_pos, is_neox, dt), start_pos)
+    orc.kv_append(want_v, v, start_pos)
+    want_q = orc.rope(q, table, start_pos, is_neox, dt)
+    d_q, d_kc, d_vc = dev_empty(q.shape), to_dev(canary_k), to_dev(canary_v)
+    ops.hip_rope_kv_append_layer(d_q, d_kc, d_vc, f32_dev(table), to_dev(q), to_dev(k), to_dev(v),
+                                 start_pos, cur_size, H, Hkv, 128, is_neox, dt)
+    assert np.array_equal(to_host(d_q), want_q)
+    assert np.array_equal(to_host(d_kc), want_k)
+    assert np.array_equal(to_host(d_vc), want_v)
+
+
+# ---------------------------------------------------------------- attention
+
+ATTN_CASES = [
+    # (m, n, offset, H, Hkv)
+    (4, 4, 0, 2, 2),
+    (3, 7, 4, 4, 2),
+    (1, 33, 32, 6, 1),
+    (17, 17, 0, 3, 1),
+    (64, 64, 0, 8, 8),
+    (65, 129, 64, 8, 2),
+    (128, 128, 0, 4, 4),
+    (200, 333, 133, 14, 2),
+    (256, 256, 0, 12, 2),
+    (300, 300, 0, 28, 4),
+    (77, 590, 513, 28, 4),
+    (513, 513, 0, 5, 5),
+]
+
+
+@pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
+@pytest.mark.parametrize("m,n,offset,H,Hkv", ATTN_CASES)
+def test_flash_attn_gqa_vs_oracle(dt, m, n, offset, H, Hkv):
+    ops = _ops()
+    seed = 1000 * m + n + H
+    q = normal_bits(seed, (m, H, 128), dt)
+    k = normal_bits(seed + 1, (n, Hkv, 128), dt)
+    v = normal_bits(seed + 2, (n, Hkv, 128), dt)
+    d_out = dev_empty(q.shape)
+    ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), m, n, offset, H // Hkv,
+                                 Hkv, 128, dt)
+    check_attention(to_host(d_out), q, k, v, n, offset, dt)
+
+
+def test_llama2_prefill_config_fp16():
+    """BASELINE config 1: Llama2-7B prefill, fp16, H = Hkv = 32, m = n = 256, through the
+    MHA entry point and the reference's own tolerance rule
+    (tests/npu_op_test_util.cpp:33-48: abs 1e-3 AND rel 1e-3)."""
+    ops = _ops()
+    dt, m, H = DT_FLOAT16, 256, 32
+    q = normal_bits(1001, (m, H, 128), dt)
+    k = normal_bits(1002, (m, H, 128), dt)
+    v = normal_bits(1003, (m, H, 128), dt)
+    for fn in (ops.hip_flash_attn_layer, ops.hip_flash_attn_opt_prefill_layer):
+        d_out = dev_empty(q.shape)
+        fn(d_out, to_dev(q), to_dev(k), to_dev(v), m, m, 0, H, 128, dt)
+        out = to_host(d_out)
+        check_attention(out, q, k, v, m, 0, dt)
+        bad, _ = orc.all_close(orc.widen(out, dt), orc.attention_f32(q, k, v, m, 0, dt))
+        assert bad == 0
+
+
+def test_llama2_decode_config_fp16():
+    """BASELINE config 2: one query token over a 512-row fp16 cache, H = Hkv = 32."""
+    ops = _ops()
+    dt, H, n = DT_FLOAT16, 32, 512
+    q = normal_bits(2001, (1, H, 128), dt)
+    k = normal_bits(2002, (n, H, 128), dt)
+    v = normal_bits(2003, (n, H, 128), dt)
+    d_out = dev_empty(q.shape)
+    ops.hip_flash_attn_layer(d_out, to_dev(q), to_dev(k), to_dev(v), 1, n, n - 1, H, 128, dt)
+    check_attention(to_host(d_out), q, k, v, n, n - 1, dt)
+
+
+@pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
+@pytest.mark.parametrize("splits", [1, 2, 3, 7, 64, 0])
+@pytest.mark.parametrize("batch,n,stride,H,Hkv", [(1, 1000, 1000, 40, 8), (3, 777, 1024, 12, 2), (2, 4096, 4096, 28, 4)])
+def test_flash_decode_splits(dt, splits, batch, n, stride, H, Hkv):
+    """Split-KV == unsplit for every split count incl. a ragged last split, batch
+    entries independent, rows beyond n never read into the result."""
+    import torch
+    ops = _ops()
+    q = normal_bits(31, (batch, 1, H, 128), dt)
+    k = normal_bits(32, (batch, stride, Hkv, 128), dt)
+    v = normal_bits(33, (batch, stride, Hkv, 128), dt)
+    # poison the rows past n with NaN bit patterns: they must not reach the output
+    k[:, n:] = 0x7FFF
+    v[:, n:] = 0x7FFF
+    g = H // Hkv
+    ns = splits if splits > 0 else ops.flash_decode_default_splits(batch, n, Hkv)
+    ws_bytes = ops.flash_decode_workspace_bytes(batch, g, Hkv, 128, ns)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+    d_out = dev_empty((batch, 1, H, 128))
+    ops.hip_flash_decode_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), ws, ws_bytes, batch, n,
+                                   stride, g, Hkv, 128, splits, dt)
+    check_attention(to_host(d_out), q, k, v, n, n - 1, dt, batch=True)
+
+
+@pytest.mark.parametrize("S,rows_per_probe", [(2400, 24), (4096, 16)])
+def test_qwen7b_prefill_full_size_sampled(S, rows_per_probe):
+    """BASELINE config 4 shape (H=28, Hkv=4, bf16) at sizes the CPU oracle cannot
+    finish whole: every sampled output row is checked against the oracle run as a
+    one-row decode over the same keys (row r of a causal prefill == decode with
+    n = r + 1)."""
+    ops = _ops()
+    dt, H, Hkv = DT_BFLOAT16, 28, 4
+    q = normal_bits(1004 + S, (S, H, 128), dt)
+    k = normal_bits(2004 + S, (S, Hkv, 128), dt)
+    v = normal_bits(3004 + S, (S, Hkv, 128), dt)
+    d_out = dev_empty(q.shape)
+    ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), S, S, 0, H // Hkv, Hkv, 128, dt)
+    out = to_host(d_out)
+    rng = np.random.default_rng(5)
+    rows = sorted(set([0, 1, 31, 32, 63, 64, 255, 256, S - 1] + list(rng.integers(0, S, rows_per_probe))))
+    worst = 0.0
+    for r in rows:
+        ref = orc.attention_f32(q[r:r + 1], k, v, r + 1, r, dt)
+        err = float(np.abs(orc.widen(out[r:r + 1], dt) - ref).max())
+        worst = max(worst, err)
+        assert err <= TOL[dt], f"row {r}: {err}"
+    assert np.isfinite(orc.widen(out, dt)).all()

@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X attention path: one JSON line on stdout.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM: the causal flash-attention prefill launch at
+BASELINE.json's Qwen2.5-7B shape (bf16, H=28, Hkv=4, head_dim 128, S=4096).
+`value` is its algorithmic throughput, 4*H*hd*S(S+1)/2 FLOP per launch over the
+measured time per launch.  The same run also measures the two other kernels of
+the path at their BASELINE shapes -- split-KV decode at the Qwen2.5-32B shape
+(H=40, Hkv=8, KV length 32768, batch 1 and 16; algorithmic bytes = K and V read
+once) and the fused RoPE + KV append -- and times the CPU oracle (a port of the
+reference's CPU layer attention, src/llama2_layer_cpu.cpp:175-296) on the host
+cores as a reported baseline.
+
+Launch durations are measured with HIP events recorded on the stream the
+kernels run on (the default stream), around back-to-back launches.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "attn prefill TFLOP/s + decode KV GB/s (Qwen2.5-7B shape), % roofline, 1 MI355X"
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+DT_BF16 = 5
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class HipTimer:
+    """Event pair on the default stream through the library's own event calls."""
+
+    def __init__(self, lib):
+        import ctypes
+        self.lib = lib
+        self.a, self.b = ctypes.c_void_p(), ctypes.c_void_p()
+        assert lib.llmhip_event_create(ctypes.byref(self.a)) == 0
+        assert lib.llmhip_event_create(ctypes.byref(self.b)) == 0
+
+    def time_ms(self, fn, reps):
+        import ctypes
+        assert self.lib.llmhip_event_record(self.a, None) == 0
+        for i in range(reps):
+            fn(i)
+        assert self.lib.llmhip_event_record(self.b, None) == 0
+        assert self.lib.llmhip_event_sync(self.b) == 0
+        ms = ctypes.c_float(0)
+        assert self.lib.llmhip_event_elapsed_ms(ctypes.byref(ms), self.a, self.b) == 0
+        return ms.value / reps
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def bench_prefill(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
+    g = torch.Generator(device="cuda").manual_seed(1004 + S)
+    q = torch.randn(S, H, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+    k = torch.randn(S, Hkv, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+    v = torch.randn(S, Hkv, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+    out = torch.empty_like(q)
+
+    def step(_):
+        ops.hip_flash_attn_gqa_layer(out, q, k, v, S, S, 0, H // Hkv, Hkv, 128, DT_BF16)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev_ms = timer.time_ms(step, steps)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    flops = 4.0 * H * 128 * S * (S + 1) / 2
+    return {"S": S, "ms_event": ev_ms, "ms_wall": wall_ms, "flops": flops,
+            "tflops": flops / (ev_ms * 1e-3) / 1e12}, (q, k, v, out)
+
+
+def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
+    """Cold numbers: successive launches walk over distinct KV buffers whose total
+    exceeds 1 GiB, so no launch is served from the 256 MB last-level cache."""
+    kv_bytes = 2 * batch * n * Hkv * 128 * 2
+    nbuf = max(2, -(-(1 << 30) // kv_bytes) + 1)
+    g = torch.Generator(device="cuda").manual_seed(1005)
+    ks, vs = [], []
+    for _ in range(nbuf):
+        ks.append(torch.randn(batch, n, Hkv, 128, device="cuda", dtype=torch.bfloat16, generator=g))
+        vs.append(torch.randn(batch, n, Hkv, 128, device="cuda", dtype=torch.bfloat16, generator=g))
+    q = torch.randn(batch, 1, H, 128, device="cuda", dtype=torch.bfloat16, generator=g)
+    out = torch.empty_like(q)
+    splits = ops.flash_decode_default_splits(batch, n, Hkv)
+    ws_bytes = ops.flash_decode_workspace_bytes(batch, H // Hkv, Hkv, 128, splits)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+
+    def step(i):
+        j = i % nbuf
+        ops.hip_flash_decode_gqa_layer(out, q, ks[j], vs[j], ws, ws_bytes, batch, n, n, H // Hkv,
+                                       Hkv, 128, splits, DT_BF16)
+
+    def hot(_):
+        ops.hip_flash_decode_gqa_layer(out, q, ks[0], vs[0], ws, ws_bytes, batch, n, n, H // Hkv,
+                                       Hkv, 128, splits, DT_BF16)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    cold = median([timer.time_ms(step, steps) for _ in range(5)])
+    hot_ms = median([timer.time_ms(hot, steps) for _ in range(3)])
+    torch.cuda.synchronize()
+    return {"batch": batch, "n": n, "splits": splits, "kv_bytes": kv_bytes, "buffers": nbuf,
+            "ms_cold": cold, "ms_hot": hot_ms, "gbs_cold": kv_bytes / (cold * 1e-3) / 1e9,
+            "gbs_hot": kv_bytes / (hot_ms * 1e-3) / 1e9}
+
+
+def bench_rope_append(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
+    import numpy as np
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q = torch.randn(S, H, 128, device="cuda", dtype=torch.bfloat16, generator=g)
+    k = torch.randn(S, Hkv, 128, device="cuda", dtype=torch.bfloat16, generator=g)
+    v = torch.randn(S, Hkv, 128, device="cuda", dtype=torch.bfloat16, generator=g)
+    oq = torch.empty_like(q)
+    kc = torch.empty(S, Hkv, 128, device="cuda", dtype=torch.bfloat16)
+    vc = torch.empty_like(kc)
+    table = torch.from_numpy(np.ascontiguousarray(ops.init_freq_cis(128, S, 1e6, DT_BF16))).cuda()
+
+    def step(_):
+        ops.hip_rope_kv_append_layer(oq, kc, vc, table, q, k, v, 0, S, H, Hkv, 128, True, DT_BF16)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ms = median([timer.time_ms(step, steps) for _ in range(3)])
+    nbytes = 2 * S * 128 * (2 * H + 4 * Hkv) + S * 64 * 8
+    return {"S": S, "ms": ms, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9}
+
+
+def cpu_baseline(S, H=28, Hkv=4):
+    """The oracle's layer-style attention (the port of the reference CPU layer
+    path) on the whole prefill workload: single thread (the reference's Eigen
+    expressions are single-threaded) and all cores."""
+    import numpy as np
+    from oracle import oracle as orc
+    rng = np.random.default_rng(1004 + S)
+    q = orc.round_to(rng.standard_normal((S, H, 128), dtype=np.float32), DT_BF16)
+    k = orc.round_to(rng.standard_normal((S, Hkv, 128), dtype=np.float32), DT_BF16)
+    v = orc.round_to(rng.standard_normal((S, Hkv, 128), dtype=np.float32), DT_BF16)
+    flops = 4.0 * H * 128 * S * (S + 1) / 2
+    cores = min(orc.max_threads(), 16)
+    t = time.perf_counter()
+    orc.attention_layer(q, k, v, S, 0, DT_BF16, n_threads=cores)
+    t_all = time.perf_counter() - t
+    t = time.perf_counter()
+    orc.attention_layer(q, k, v, S, 0, DT_BF16, n_threads=1)
+    t_one = time.perf_counter() - t
+    return {"value": flops / t_all / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"whole prefill workload (S={S}, H={H}, Hkv={Hkv}, bf16, {flops / 1e9:.1f} GFLOP), "
+                      f"layer-style oracle: {t_all:.2f} s on {cores} threads, {t_one:.2f} s on 1 thread",
+            "single_thread_value": flops / t_one / 1e12, "seconds_all_cores": t_all,
+            "seconds_single_thread": t_one}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--seq", type=int, default=4096, help="prefill sequence length of the timed step")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="comma list of legs: prefill,decode,rope (default all)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build measures one GPU; --gpus must be 1 "
+            "(the path shards by kv head without any exchange, see DESIGN.md)")
+        sys.exit(2)
+
+    import torch
+    import llm_simple_amd.ops as ops
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible")
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    timer = HipTimer(ops.lib)
+    legs = set(args.only.split(",")) if args.only else {"prefill", "decode", "rope"}
+    extra = {}
+
+    # ---- the timed step: prefill at the headline shape ----
+    torch.cuda.synchronize()
+    pre, _ = bench_prefill(ops, torch, timer, args.seq, args.steps, args.warmup)
+    log(f"prefill S={args.seq}: {pre['ms_event'] * 1e3:.1f} us  {pre['tflops']:.1f} TFLOP/s")
+    if "prefill" in legs:
+        others = []
+        for S in (1024, 8192):
+            if S == args.seq:
+                continue
+            r, _ = bench_prefill(ops, torch, timer, S, max(10, args.steps // 4), 5)
+            log(f"prefill S={S}: {r['ms_event'] * 1e3:.1f} us  {r['tflops']:.1f} TFLOP/s")
+            others.append({"S": S, "us": r["ms_event"] * 1e3, "tflops": r["tflops"],
+                           "frac": r["tflops"] / PEAK_BF16_TFLOPS})
+        extra["prefill_other"] = others
+
+    if "decode" in legs:
+        dec = []
+        for batch, n in ((16, 32768), (1, 32768), (1, 4096), (1, 16384), (16, 4096), (16, 16384)):
+            r = bench_decode(ops, torch, timer, batch, n, max(20, args.steps // 2), 10)
+            log(f"decode B={batch} n={n} splits={r['splits']}: cold {r['ms_cold'] * 1e3:.1f} us "
+                f"{r['gbs_cold']:.0f} GB/s, hot {r['ms_hot'] * 1e3:.1f} us {r['gbs_hot']:.0f} GB/s")
+            dec.append(r)
+            torch.cuda.empty_cache()
+        head = dec[0]
+        extra["decode_value"] = head["gbs_cold"]
+        extra["decode_unit"] = "GB/s"
+        extra["roofline_decode"] = {
+            "bound": "hbm", "achieved": head["gbs_cold"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": head["gbs_cold"] / PEAK_HBM_GBS, "traffic": None,
+            "workload": "Qwen2.5-32B decode bf16 H=40 Hkv=8 n=32768 batch=16 (2 GiB of K+V per launch, cold)"}
+        extra["decode_all"] = [
+            {"batch": r["batch"], "n": r["n"], "splits": r["splits"], "us_cold": r["ms_cold"] * 1e3,
+             "gbs_cold": r["gbs_cold"], "frac_cold": r["gbs_cold"] / PEAK_HBM_GBS,
+             "us_hot": r["ms_hot"] * 1e3, "gbs_hot": r["gbs_hot"]} for r in dec]
+
+    if "rope" in legs:
+        r = bench_rope_append(ops, torch, timer, args.seq, max(20, args.steps // 2), 10)
+        log(f"rope+append S={args.seq}: {r['ms'] * 1e3:.1f} us {r['gbs']:.0f} GB/s")
+        extra["rope_kv_append"] = {"S": r["S"], "us": r["ms"] * 1e3, "gbs": r["gbs"],
+                                   "frac": r["gbs"] / PEAK_HBM_GBS}
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(args.seq)
+        log(f"cpu baseline: {cpu['sample']}")
+
+    line = {
+        "metric": METRIC,
+        "value": pre["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": pre["ms_wall"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"Qwen2.5-7B causal prefill attention, bf16, batch 1, H=28, Hkv=4, "
+                               f"head_dim=128, S={args.seq} (BASELINE configs[3]); decode leg: "
+                               f"Qwen2.5-32B H=40 Hkv=8 n=32768 (configs[4])"},
+        "roofline": {"bound": "mfma", "achieved": pre["tflops"], "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": pre["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "flash_prefill_kernel<bf16>", "us_per_launch": pre["ms_event"] * 1e3,
+                     "flops_per_launch": pre["flops"]},
+        "cpu_baseline": cpu,
+    }
+    line.update(extra)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -243,24 +243,60 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
   }
 }
 
-// grid (rows, Hkv, batch), 128 threads: thread d folds the splits of one
-// output row with the log-sum-exp rule.
+// grid (rows, Hkv, batch), 128 threads: folds the splits of one output row with
+// the log-sum-exp rule.  The per-split (max, sum) pairs are read once, in
+// parallel, into LDS; thread d then accumulates its column with independent
+// loads in flight.
+constexpr int kMaxSplits = 256;
+
 template <typename T>
 __global__ __launch_bounds__(128) void flash_decode_combine_kernel(DecodeParams p) {
   using E = Elem<T>;
+  __shared__ float w_s[kMaxSplits];
+  __shared__ float red[4];
   const int c = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int d = threadIdx.x;
-  const size_t base = ((size_t)b * p.Hkv + kvh) * p.num_splits;
-  float M = -INFINITY;
-  for (int s = 0; s < p.num_splits; ++s) M = fmaxf(M, p.ws_ml[((base + s) * kDecCols + c) * 2]);
-  const float M_use = (M == -INFINITY) ? 0.0f : M;
-  float L = 0.0f, acc = 0.0f;
-  for (int s = 0; s < p.num_splits; ++s) {
-    const size_t slot = (base + s) * kDecCols + c;
-    const float wt = fast_exp2(p.ws_ml[slot * 2] - M_use);
-    L += wt * p.ws_ml[slot * 2 + 1];
-    acc += wt * p.ws_o[slot * kHeadDim + d];
+  const int S = p.num_splits;
+  const size_t base = ((size_t)b * p.Hkv + kvh) * S;
+  // pass 1: this thread owns splits d and d + 128
+  float m0 = -INFINITY, m1 = -INFINITY, l0 = 0.0f, l1 = 0.0f;
+  if (d < S) {
+    m0 = p.ws_ml[((base + d) * kDecCols + c) * 2];
+    l0 = p.ws_ml[((base + d) * kDecCols + c) * 2 + 1];
   }
+  if (d + 128 < S) {
+    m1 = p.ws_ml[((base + d + 128) * kDecCols + c) * 2];
+    l1 = p.ws_ml[((base + d + 128) * kDecCols + c) * 2 + 1];
+  }
+  float M = fmaxf(m0, m1);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+  if ((d & 63) == 0) red[d >> 6] = M;
+  __syncthreads();
+  M = fmaxf(red[0], red[1]);
+  const float M_use = (M == -INFINITY) ? 0.0f : M;
+  const float w0 = fast_exp2(m0 - M_use), w1 = fast_exp2(m1 - M_use);
+  if (d < S) w_s[d] = w0;
+  if (d + 128 < S) w_s[d + 128] = w1;
+  float L = w0 * l0 + w1 * l1;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+  if ((d & 63) == 0) red[2 + (d >> 6)] = L;
+  __syncthreads();
+  L = red[2] + red[3];
+  // pass 2: weighted sum of the partial outputs
+  const float *src = p.ws_o + (base * kDecCols + c) * kHeadDim + d;
+  const size_t stride = (size_t)kDecCols * kHeadDim;
+  float acc = 0.0f;
+  int s = 0;
+  for (; s + 8 <= S; s += 8) {
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = src[(size_t)(s + j) * stride];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc += w_s[s + j] * x[j];
+  }
+  for (; s < S; ++s) acc += w_s[s] * src[(size_t)s * stride];
   const float inv = (L > 0.0f) ? 1.0f / L : 0.0f;
   const int r = c / p.g, hq = c % p.g;
   uint16_t *op = reinterpret_cast<uint16_t *>(

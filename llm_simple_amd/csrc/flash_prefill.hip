@@ -6,28 +6,32 @@
 // (src/llama2_layer_cpu.cpp:687-701), scale = 1/sqrt(128) inside
 // (src/llama2_layer_cpu.cpp:177), query head h reading kv head h / group_size.
 //
-// Work decomposition.  One workgroup = 4 wavefronts = one (query tile, query
-// head).  A query tile is 4*QB blocks of 32 rows; wave w owns blocks {w} (QB=1)
-// or {w, 7-w} (QB=2) so that the causal diagonal costs every wave the same.
-// The workgroup walks the visible keys in tiles of 64; K and V tiles are staged
-// in LDS (double buffered, XOR-swizzled 256-byte rows) by all 256 threads with
-// 128-bit loads and are shared by the four waves.
+// Common to both kernels below.  A wave owns 32 query rows.  The scores are
+// produced transposed, S^T = K Q^T, with mfma_f32_32x32x16: every lane then
+// holds 16 keys of ONE query column per 32-key block, so the softmax row
+// reductions are in-register plus one exchange with lane^32
+// (v_permlane32_swap).  The probabilities, rounded to the storage type, are
+// already laid out as the B operand of O^T += V^T P^T (the contraction index is
+// permuted consistently on the V side), so P never touches LDS.  K and V tiles
+// of 64 keys are staged in LDS, XOR-swizzled 256-byte rows; K fragments are
+// read with ds_read_b128, V^T fragments with ds_read_b64_tr_b16.  exp2 with the
+// scale folded into one FMA; the running maximum is kept in raw score units; O
+// is rescaled only when some row's maximum moved.  Accumulation is fp32; out =
+// O / l rounded once; l sums the ROUNDED probabilities (what P.V used).
 //
-// Per wave and tile the scores are produced transposed, S^T = K Q^T, with
-// mfma_f32_32x32x16: every lane then holds 16 keys of ONE query column, so the
-// softmax row reductions are in-register plus one exchange with lane^32.  The
-// probabilities, rounded to the storage type, are already laid out as the B
-// operand of O^T += V^T P^T (the contraction index is permuted consistently on
-// the V side), so P never touches LDS.  V^T fragments come from
-// ds_read_b64_tr_b16.  Accumulation is fp32; out = O / l rounded once.
+// flash_prefill_kernel      4 waves, 128 query rows, two workgroups per CU:
+//                           used when the problem has few query tiles.
+// flash_prefill_pp_kernel   8 waves, 256 query rows, one workgroup per CU, two
+//                           groups of 4 waves running half an iteration apart
+//                           (one group's MFMA phase against the other group's
+//                           softmax phase), K/V tiles shared by all 8 waves.
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace llmhip {
 
-constexpr int kTileN = 64;                        // keys per LDS tile
-constexpr int kTileBytes = kTileN * kRowBytes;    // 16 KiB
-constexpr int kPrefillThreads = 256;
+constexpr int kTileN = 64;                      // keys per LDS tile
+constexpr int kTileBytes = kTileN * kRowBytes;  // 16 KiB
 
 struct PrefillParams {
   const char *q;
@@ -73,233 +77,396 @@ __device__ __forceinline__ bool prefill_schedule(const PrefillParams &p, int bid
   return true;
 }
 
-template <typename T, int QB>
-__global__ __launch_bounds__(kPrefillThreads) void flash_prefill_kernel(PrefillParams p) {
+// max / sum over the lane pair (l, l^32) without going through the LDS
+// crossbar.  v_permlane32_swap(a, b) exchanges a[32..63] with b[0..31]; with
+// a == b == x the two results are (x_lo, x_lo) and (x_hi, x_hi).  The results
+// are copied to scalars before the bit cast: a bit cast applied directly to a
+// vector element reads element 0.
+__device__ __forceinline__ void pair_swap(float x, float &lo, float &hi) {
+  typedef __attribute__((ext_vector_type(2))) unsigned u2;
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const u2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  lo = __builtin_bit_cast(float, r0);
+  hi = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float pair_max(float x) {
+  float lo, hi;
+  pair_swap(x, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  float lo, hi;
+  pair_swap(x, lo, hi);
+  return lo + hi;
+}
+
+// acc + lo + hi of a packed pair of storage-type values.
+template <typename T> __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc);
+template <> __device__ __forceinline__ float dot2_ones<__bf16>(uint32_t packed, float acc) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 b2;
+  const b2 one = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, packed), one, acc, false);
+}
+template <> __device__ __forceinline__ float dot2_ones<_Float16>(uint32_t packed, float acc) {
+  typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+  const h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), one, acc, false);
+}
+
+// LDS visibility + workgroup barrier that does not drain outstanding global loads.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// State of one wave: 32 query rows (one per lane pair), fp32 O^T accumulators.
+template <typename T> struct WaveAttn {
   using E = Elem<T>;
-  constexpr int BM = 4 * QB * 32;
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  // lds: [2 stages][K tile | V tile]
+  f32x16_t o[4];       // O^T: d block x (16 d rows of this lane)
+  f32x16_t s[2];       // S^T / P^T of the current tile: key block x 16 keys
+  u32x4_t pf[2][2];    // P^T packed as B operand: key block x k-step
+  u32x4_t qf[8];       // Q^T fragments (B operand), loaded once
+  float m_run, l_run;  // running max (raw score units) and sum of this lane's keys
+  int lane, l32, hh, g16, li;
+
+  __device__ __forceinline__ void init(int lane_) {
+    lane = lane_;
+    l32 = lane & 31;
+    hh = lane >> 5;
+    g16 = lane >> 4;
+    li = lane & 15;
+    m_run = -INFINITY;
+    l_run = 0.0f;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[d][i] = 0.0f;
+  }
+
+  __device__ __forceinline__ void load_q(const char *q_row_head) {
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) qf[kk] = global_load_b128(q_row_head + hh * 16 + kk * 32);
+  }
+  // The Q loads are complete after this: no wait inside the key loop is ever
+  // attributed to them.
+  __device__ __forceinline__ void pin_q() {
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) asm volatile("" : "+v"(qf[kk]));
+  }
+
+  // S^T = K Q^T for the 64 keys of the tile at ks.
+  __device__ __forceinline__ void qk(const char *ks) {
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const u32x4_t kf = lds_read_b128(ks, k_swizzle_off(kb * 32 + l32, 2 * kk + hh));
+        if (kk == 0) {
+          f32x16_t z;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) z[i] = 0.0f;
+          s[kb] = E::mfma32(kf, qf[kk], z);
+        } else {
+          s[kb] = E::mfma32(kf, qf[kk], s[kb]);
+        }
+      }
+    }
+  }
+
+  // O^T += V^T P^T.  Lane (d = 32*dblk + l32, hh): element e of k-step (kb, ks2)
+  // is the key 32*kb + 16*ks2 + 8*(e/4) + 4*hh + e%4 -- the key P's element e
+  // carries.
+  __device__ __forceinline__ void pv(const char *vs) {
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int ks2 = 0; ks2 < 2; ++ks2) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const int kr0 = kb * 32 + ks2 * 16 + 4 * hh + (li >> 2);
+          const int gran = d * 4 + (g16 & 1) * 2 + ((li & 3) >> 1);
+          const int sub = (li & 1) * 8;
+          const u32x2_t lo = lds_read_tr16(vs, v_swizzle_off(kr0, gran) + sub);
+          const u32x2_t hi = lds_read_tr16(vs, v_swizzle_off(kr0 + 8, gran) + sub);
+          const u32x4_t vf = {lo[0], lo[1], hi[0], hi[1]};
+          o[d] = E::mfma32(vf, pf[kb][ks2], o[d]);
+        }
+      }
+  }
+
+  // Online softmax of s -> pf.  qrow: query row of this lane's column; rows see
+  // keys <= qrow + offset; `partial` says whether any key of the tile can be
+  // masked for any row of the wave.
+  __device__ __forceinline__ void softmax(int key0, int qrow, int offset, int n, bool partial,
+                                          float scale_log2e) {
+    if (partial) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = key0 + kb * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+          if (key > qrow + offset || key >= n) s[kb][i] = -INFINITY;
+        }
+    }
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kb][i]);
+    mloc = pair_max(mloc);
+    const float m_new = fmaxf(m_run, mloc);
+    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+    const float neg_ms = -m_use * scale_log2e;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        s[kb][i] = fast_exp2(__builtin_fmaf(s[kb][i], scale_log2e, neg_ms));
+    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+      const float alpha = fast_exp2((m_run - m_use) * scale_log2e);
+      l_run *= alpha;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+    }
+    m_run = m_new;
+    float ps0 = 0.0f, ps1 = 0.0f;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int ks2 = 0; ks2 < 2; ++ks2) {
+        u32x4_t w;
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          w[e2] = E::pack2(s[kb][8 * ks2 + 2 * e2], s[kb][8 * ks2 + 2 * e2 + 1]);
+          if (e2 & 1)
+            ps1 = dot2_ones<T>(w[e2], ps1);
+          else
+            ps0 = dot2_ones<T>(w[e2], ps0);
+        }
+        pf[kb][ks2] = w;
+      }
+    l_run += ps0 + ps1;
+  }
+
+  // out[qrow][head][d] = O^T / l, rounded once.
+  __device__ __forceinline__ void store(char *out_row_head, bool valid) {
+    const float l_tot = pair_sum(l_run);
+    const float inv = (l_tot > 0.0f) ? 1.0f / l_tot : 0.0f;
+    if (!valid) return;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        u32x2_t w;
+        w[0] = E::pack2(o[d][4 * i4] * inv, o[d][4 * i4 + 1] * inv);
+        w[1] = E::pack2(o[d][4 * i4 + 2] * inv, o[d][4 * i4 + 3] * inv);
+        const int dd = 32 * d + 8 * i4 + 4 * hh;
+        *reinterpret_cast<u32x2_t *>(out_row_head + dd * 2) = w;
+      }
+  }
+};
+
+// Cooperative K or V tile loader for NT threads: thread -> row t/16 (+ NT/16 per
+// index i), 16-byte granule t%16.  The per-thread byte offset is loop invariant
+// and the tile base is wave uniform, so a full tile costs no address arithmetic;
+// only the tile that straddles row n clamps its keys.
+template <int NT> struct TileLoader {
+  static constexpr int kPer = 1024 / NT;  // granules per thread per tile
+  static constexpr int kRowStep = NT / 16;
+  int row, gi, n;
+  uint32_t off;
+  size_t kv_row_bytes;
+  __device__ __forceinline__ void init(int t, size_t kv_row_bytes_, int n_) {
+    row = t >> 4;
+    gi = t & 15;
+    n = n_;
+    kv_row_bytes = kv_row_bytes_;
+    off = (uint32_t)row * (uint32_t)kv_row_bytes_ + (uint32_t)gi * 16u;
+  }
+  __device__ __forceinline__ void load(const char *base, int t, u32x4_t (&r)[kPer]) const {
+    if ((t + 1) * kTileN <= n) {
+      const char *b_ = base + (size_t)t * kTileN * kv_row_bytes;
+#pragma unroll
+      for (int i = 0; i < kPer; ++i)
+        r[i] = global_load_b128(b_ + (size_t)i * kRowStep * kv_row_bytes + off);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kPer; ++i) {
+        const int key = min(t * kTileN + row + kRowStep * i, n - 1);
+        r[i] = global_load_b128(base + (size_t)key * kv_row_bytes + gi * 16);
+      }
+    }
+  }
+  __device__ __forceinline__ void store_k(char *stage, const u32x4_t (&r)[kPer]) const {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i)
+      lds_write_b128(stage, k_swizzle_off(row + kRowStep * i, gi), r[i]);
+  }
+  __device__ __forceinline__ void store_v(char *stage, const u32x4_t (&r)[kPer]) const {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i)
+      lds_write_b128(stage, v_swizzle_off(row + kRowStep * i, gi), r[i]);
+  }
+};
+
+// ---------------------------------------------------------------------------
+// 4 waves, 128 query rows, double-buffered K/V tiles, two workgroups per CU.
+// ---------------------------------------------------------------------------
+constexpr int kSmallThreads = 256;
+constexpr int kSmallBM = 128;
+
+template <typename T>
+__global__ __launch_bounds__(kSmallThreads, 2) void flash_prefill_kernel(PrefillParams p) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // [2 stages][K tile | V tile]
   int tile, head;
   if (!prefill_schedule(p, blockIdx.x, tile, head)) return;
 
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6;
-  const int lane = tid & 63;
-  const int l32 = lane & 31;
-  const int hh = lane >> 5;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int kvh = head / p.g;
-  const int row0 = tile * BM;
-  const int rows_end = min(p.m, row0 + BM);
-  // keys any row of this tile can see
-  const int n_vis = min(p.n, rows_end + p.offset);
-  const int num_tiles = (n_vis + kTileN - 1) / kTileN;
-
+  const int row0 = tile * kSmallBM;
+  const int rows_end = min(p.m, row0 + kSmallBM);
+  const int n_vis = min(p.n, rows_end + p.offset);  // keys any row of this tile can see
+  const int J = (n_vis + kTileN - 1) / kTileN;
   const size_t q_row_bytes = (size_t)p.H * kRowBytes;
   const size_t kv_row_bytes = (size_t)p.Hkv * kRowBytes;
   const char *kbase = p.k + (size_t)kvh * kRowBytes;
   const char *vbase = p.v + (size_t)kvh * kRowBytes;
 
-  // ---- this wave's query blocks and Q^T fragments (B operand) ----
-  int qrow[QB];     // query row of this lane's column
-  int qblk0[QB];    // first row of the block
-  u32x4_t qf[QB][8];
-#pragma unroll
-  for (int b = 0; b < QB; ++b) {
-    const int blk = (b == 0) ? wave : (4 * QB - 1 - wave);
-    qblk0[b] = row0 + blk * 32;
-    qrow[b] = qblk0[b] + l32;
-    const int rr = min(qrow[b], p.m - 1);
-    const char *qp = p.q + (size_t)rr * q_row_bytes + (size_t)head * kRowBytes + hh * 16;
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) qf[b][kk] = global_load_b128(qp + kk * 32);
-  }
+  WaveAttn<T> w;
+  w.init(lane);
+  const int qblk0 = row0 + wave * 32;
+  const int qrow = qblk0 + w.l32;
+  const int last_row = min(qblk0 + 31, p.m - 1);
+  const int Jw = (qblk0 < p.m) ? min(J, (min(p.n, last_row + p.offset + 1) + kTileN - 1) / kTileN) : 0;
+  w.load_q(p.q + (size_t)min(qrow, p.m - 1) * q_row_bytes + (size_t)head * kRowBytes);
 
-  f32x16_t o[QB][4];
-  float m_run[QB], l_run[QB];
-#pragma unroll
-  for (int b = 0; b < QB; ++b) {
-    m_run[b] = -INFINITY;
-    l_run[b] = 0.0f;
-#pragma unroll
-    for (int d = 0; d < 4; ++d)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[b][d][i] = 0.0f;
-  }
-
-  // ---- cooperative tile loader: thread -> 4 granules of K and 4 of V ----
+  TileLoader<kSmallThreads> ld;
+  ld.init(tid, kv_row_bytes, p.n);
   u32x4_t kreg[4], vreg[4];
-  auto load_tile_regs = [&](int j) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * kPrefillThreads;
-      const int r = c >> 4, gi = c & 15;
-      const int key = min(j * kTileN + r, p.n - 1);
-      const size_t off = (size_t)key * kv_row_bytes + gi * 16;
-      kreg[i] = global_load_b128(kbase + off);
-      vreg[i] = global_load_b128(vbase + off);
-    }
-  };
-  auto store_tile_lds = [&](int stage) {
-    char *ks = lds + stage * 2 * kTileBytes;
+  ld.load(kbase, 0, kreg);
+  ld.load(vbase, 0, vreg);
+  ld.store_k(lds, kreg);
+  ld.store_v(lds + kTileBytes, vreg);
+  w.pin_q();
+  lds_barrier();
+
+  for (int j = 0; j < J; ++j) {
+    char *ks = lds + (j & 1) * 2 * kTileBytes;
     char *vs = ks + kTileBytes;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * kPrefillThreads;
-      const int r = c >> 4, gi = c & 15;
-      lds_write_b128(ks, k_swizzle_off(r, gi), kreg[i]);
-      lds_write_b128(vs, v_swizzle_off(r, gi), vreg[i]);
+    char *ks_next = lds + ((j + 1) & 1) * 2 * kTileBytes;
+    const int jn = min(j + 1, J - 1);  // the last prefetch is redundant but branch free
+    ld.load(kbase, jn, kreg);
+    ld.load(vbase, jn, vreg);
+    if (j < Jw) {
+      const int key0 = j * kTileN;
+      const bool partial = (key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n);
+      w.qk(ks);
+      w.softmax(key0, qrow, p.offset, p.n, partial, p.scale_log2e);
+      w.pv(vs);
     }
-  };
-
-  if (num_tiles > 0) {
-    load_tile_regs(0);
-    store_tile_lds(0);
+    ld.store_k(ks_next, kreg);
+    ld.store_v(ks_next + kTileBytes, vreg);
+    lds_barrier();
   }
-  __syncthreads();
-
-  for (int j = 0; j < num_tiles; ++j) {
-    const int stage = j & 1;
-    const bool has_next = (j + 1) < num_tiles;
-    if (has_next) load_tile_regs(j + 1);
-
-    const char *ks = lds + stage * 2 * kTileBytes;
-    const char *vs = ks + kTileBytes;
-    const int key0 = j * kTileN;
-
-    // which of this wave's query blocks see any key of this tile
-    bool active[QB], partial[QB];
-    bool any_active = false;
-#pragma unroll
-    for (int b = 0; b < QB; ++b) {
-      const int last_row = min(qblk0[b] + 31, p.m - 1);
-      active[b] = (qblk0[b] < p.m) && (key0 <= last_row + p.offset);
-      partial[b] = (key0 + kTileN - 1 > qblk0[b] + p.offset) || (key0 + kTileN > p.n);
-      any_active |= active[b];
-    }
-
-    if (any_active) {
-      // ---- S^T = K Q^T ----
-      f32x16_t s[QB][2];
-#pragma unroll
-      for (int b = 0; b < QB; ++b)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) s[b][kb][i] = 0.0f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const int r = kb * 32 + l32;
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-          const u32x4_t kf = lds_read_b128(ks, k_swizzle_off(r, 2 * kk + hh));
-#pragma unroll
-          for (int b = 0; b < QB; ++b)
-            if (active[b]) s[b][kb] = E::mfma32(kf, qf[b][kk], s[b][kb]);
-        }
-      }
-
-      // ---- online softmax per query column, P packed as B operand ----
-      u32x4_t pf[QB][2][2];
-#pragma unroll
-      for (int b = 0; b < QB; ++b) {
-        if (!active[b]) continue;
-        float mloc = -INFINITY;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            float t = s[b][kb][i] * p.scale_log2e;
-            if (partial[b]) {
-              const int key = key0 + kb * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-              if (key > qrow[b] + p.offset || key >= p.n) t = -INFINITY;
-            }
-            s[b][kb][i] = t;
-            mloc = fmaxf(mloc, t);
-          }
-        mloc = fmaxf(mloc, xor_lane(mloc, 32));
-        const float m_new = fmaxf(m_run[b], mloc);
-        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float alpha = fast_exp2(m_run[b] - m_use);
-        m_run[b] = m_new;
-        float psum = 0.0f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const float e = fast_exp2(s[b][kb][i] - m_use);
-            s[b][kb][i] = e;
-            psum += e;
-          }
-        l_run[b] = l_run[b] * alpha + psum;
-#pragma unroll
-        for (int d = 0; d < 4; ++d)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[b][d][i] *= alpha;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int ks2 = 0; ks2 < 2; ++ks2) {
-            u32x4_t w;
-#pragma unroll
-            for (int e2 = 0; e2 < 4; ++e2)
-              w[e2] = E::pack2(s[b][kb][8 * ks2 + 2 * e2], s[b][kb][8 * ks2 + 2 * e2 + 1]);
-            pf[b][kb][ks2] = w;
-          }
-      }
-
-      // ---- O^T += V^T P^T ----
-      // lane (d = 32*dblk + l32, hh): element e of k-step (kb, ks2) is the key
-      // 32*kb + 16*ks2 + 8*(e/4) + 4*hh + e%4 -- the key P's element e carries.
-      const int grp = lane >> 4;       // 16-lane group: d half = grp&1, hh = grp>>1
-      const int li = lane & 15;
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int ks2 = 0; ks2 < 2; ++ks2) {
-            const int kr0 = kb * 32 + ks2 * 16 + 4 * hh + (li >> 2);
-            const int gran = d * 4 + (grp & 1) * 2 + ((li & 3) >> 1);
-            const int sub = (li & 1) * 8;
-            const u32x2_t lo = lds_read_tr16(vs, v_swizzle_off(kr0, gran) + sub);
-            const u32x2_t hi = lds_read_tr16(vs, v_swizzle_off(kr0 + 8, gran) + sub);
-            const u32x4_t vf = {lo[0], lo[1], hi[0], hi[1]};
-#pragma unroll
-            for (int b = 0; b < QB; ++b)
-              if (active[b]) o[b][d] = E::mfma32(vf, pf[b][kb][ks2], o[b][d]);
-          }
-      }
-    }
-
-    if (has_next) store_tile_lds(stage ^ 1);
-    __syncthreads();
-  }
-
-  // ---- epilogue: out[q][head][d] = O^T / l ----
-#pragma unroll
-  for (int b = 0; b < QB; ++b) {
-    const float l_tot = l_run[b] + xor_lane(l_run[b], 32);
-    const float inv = (l_tot > 0.0f) ? 1.0f / l_tot : 0.0f;
-    if (qrow[b] < p.m) {
-      char *op = p.out + (size_t)qrow[b] * q_row_bytes + (size_t)head * kRowBytes;
-#pragma unroll
-      for (int d = 0; d < 4; ++d)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          u32x2_t w;
-          w[0] = E::pack2(o[b][d][4 * i4] * inv, o[b][d][4 * i4 + 1] * inv);
-          w[1] = E::pack2(o[b][d][4 * i4 + 2] * inv, o[b][d][4 * i4 + 3] * inv);
-          const int dd = 32 * d + 8 * i4 + 4 * hh;
-          *reinterpret_cast<u32x2_t *>(op + dd * 2) = w;
-        }
-    }
-  }
+  w.store(p.out + (size_t)qrow * q_row_bytes + (size_t)head * kRowBytes, qrow < p.m);
 }
 
-template <typename T, int QB>
+// ---------------------------------------------------------------------------
+// 8 waves, 256 query rows, two groups of 4 waves half an iteration apart.
+//
+// Phases are separated by workgroup barriers and numbered globally: group 0
+// runs its MFMA work for tile `it` (P.V of tile it-1, then S = K Q^T of tile it)
+// in phase 2it and the softmax of tile it in phase 2it+1; group 1 does the same
+// one phase later, so each phase pairs one group's MFMAs with the other group's
+// VALU work.  K(t) is read in phases 2t and 2t+1, V(t) in phases 2t+2 and 2t+3,
+// each from a two-stage ring.  Group 0 loads K(it+1) at the start of phase 2it
+// and stores it to LDS at the end of phase 2it+1 (first read in 2it+2); group 1
+// loads V(it+1) at the start of phase 2it+2 and stores it at the end of phase
+// 2it+3 (first read in 2it+4).  Both overwrite a stage whose last reader
+// finished two barriers earlier.
+// ---------------------------------------------------------------------------
+constexpr int kPPThreads = 512;
+constexpr int kPPBM = 256;
+
+template <typename T>
+__global__ __launch_bounds__(kPPThreads, 1) void flash_prefill_pp_kernel(PrefillParams p) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // K0 | K1 | V0 | V1
+  int tile, head;
+  if (!prefill_schedule(p, blockIdx.x, tile, head)) return;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int grp = wave >> 2;
+  const int kvh = head / p.g;
+  const int row0 = tile * kPPBM;
+  const int rows_end = min(p.m, row0 + kPPBM);
+  const int n_vis = min(p.n, rows_end + p.offset);
+  const int J = (n_vis + kTileN - 1) / kTileN;  // >= 1
+  const size_t q_row_bytes = (size_t)p.H * kRowBytes;
+  const size_t kv_row_bytes = (size_t)p.Hkv * kRowBytes;
+  const char *kbase = p.k + (size_t)kvh * kRowBytes;
+  const char *vbase = p.v + (size_t)kvh * kRowBytes;
+  char *const kst = lds;
+  char *const vst = lds + 2 * kTileBytes;
+
+  WaveAttn<T> w;
+  w.init(lane);
+  // query block (wave&3)*2 + grp: both groups see the same mix of diagonal work
+  const int qblk0 = row0 + ((wave & 3) * 2 + grp) * 32;
+  const int qrow = qblk0 + w.l32;
+  const int last_row = min(qblk0 + 31, p.m - 1);
+  const int Jw = (qblk0 < p.m) ? min(J, (min(p.n, last_row + p.offset + 1) + kTileN - 1) / kTileN) : 0;
+  w.load_q(p.q + (size_t)min(qrow, p.m - 1) * q_row_bytes + (size_t)head * kRowBytes);
+
+  TileLoader<256> ld;  // one group loads a whole tile
+  ld.init(tid & 255, kv_row_bytes, p.n);
+  u32x4_t rr[4];
+  {  // prologue: K(0), V(0) by group 0; K(1) by group 1
+    u32x4_t r2[4];
+    if (grp == 0) {
+      ld.load(kbase, 0, rr);
+      ld.load(vbase, 0, r2);
+      ld.store_k(kst, rr);
+      ld.store_v(vst, r2);
+    } else if (J > 1) {
+      ld.load(kbase, 1, rr);
+      ld.store_k(kst + kTileBytes, rr);
+    }
+  }
+  w.pin_q();
+  lds_barrier();
+
+  if (grp == 1) lds_barrier();
+  for (int it = 0; it <= J; ++it) {
+    // ---- MFMA phase ----
+    if (grp == 0 && it >= 1 && it + 1 < J) ld.load(kbase, it + 1, rr);
+    __builtin_amdgcn_s_setprio(2);
+    if (it >= 1 && it - 1 < Jw) w.pv(vst + ((it - 1) & 1) * kTileBytes);
+    if (it < Jw) w.qk(kst + (it & 1) * kTileBytes);
+    __builtin_amdgcn_s_setprio(0);
+    if (grp == 1 && it >= 1 && it < J) ld.store_v(vst + (it & 1) * kTileBytes, rr);
+    lds_barrier();
+    // ---- softmax phase ----
+    if (grp == 1 && it + 1 < J) ld.load(vbase, it + 1, rr);
+    if (it < Jw) {
+      const int key0 = it * kTileN;
+      const bool partial = (key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n);
+      w.softmax(key0, qrow, p.offset, p.n, partial, p.scale_log2e);
+    }
+    if (grp == 0 && it >= 1 && it + 1 < J) ld.store_k(kst + ((it + 1) & 1) * kTileBytes, rr);
+    lds_barrier();
+  }
+  if (grp == 0) lds_barrier();
+
+  w.store(p.out + (size_t)qrow * q_row_bytes + (size_t)head * kRowBytes, qrow < p.m);
+}
+
+template <typename T, bool PP>
 static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) {
   PrefillParams p = p0;
-  constexpr int BM = 4 * QB * 32;
+  constexpr int BM = PP ? kPPBM : kSmallBM;
+  constexpr int NT = PP ? kPPThreads : kSmallThreads;
   p.num_q_tiles = (p.m + BM - 1) / BM;
   const int T_ = p.num_q_tiles;
   int grid;
@@ -317,8 +484,8 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
     p.sched_a = 0;
     grid = T_ * p.H;
   }
-  const size_t lds_bytes = 2 * 2 * kTileBytes;
-  auto kern = flash_prefill_kernel<T, QB>;
+  const size_t lds_bytes = 4 * kTileBytes;
+  void (*kern)(PrefillParams) = PP ? flash_prefill_pp_kernel<T> : flash_prefill_kernel<T>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -327,7 +494,7 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kPrefillThreads), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds_bytes, stream, p);
   return hipGetLastError();
 }
 
@@ -346,12 +513,12 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
   p.Hkv = kv_head_num;
   p.H = group_size * kv_head_num;
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
-  // Small problems: 128-row tiles give more workgroups; large ones: 256-row
-  // tiles halve the LDS traffic per flop.
-  const bool big = (long long)((m + 255) / 256) * p.H >= 256;
+  // 256-row workgroups once they alone fill the 256 CUs; 128-row ones (two per
+  // CU) for smaller problems.
+  const bool pp = (long long)((m + kPPBM - 1) / kPPBM) * p.H >= 256;
   if (dt == kDtFloat16)
-    return big ? launch_prefill_t<_Float16, 2>(p, stream) : launch_prefill_t<_Float16, 1>(p, stream);
-  return big ? launch_prefill_t<__bf16, 2>(p, stream) : launch_prefill_t<__bf16, 1>(p, stream);
+    return pp ? launch_prefill_t<_Float16, true>(p, stream) : launch_prefill_t<_Float16, false>(p, stream);
+  return pp ? launch_prefill_t<__bf16, true>(p, stream) : launch_prefill_t<__bf16, false>(p, stream);
 }
 
 }  // namespace llmhip

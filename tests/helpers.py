@@ -49,10 +49,11 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None):
 
     Against the fp32 oracle (the reference's test golden): max-abs <= TOL, the
     bar BASELINE sets.  Against the layer-style oracle, whose output is itself
-    rounded to the storage type and, for bf16, sits up to ~1e-2 from the fp32
-    oracle on rows that see few keys (tests/test_oracle_attention.py): within
-    TOL, or within two representable steps of it (one bf16 step at |x| >= 2 is
-    already 1.6e-2)."""
+    rounded to the storage type: fp16 (the arithmetic the reference's CPU layer
+    really has) within TOL or two representable steps; bf16 (no reference code,
+    the same chain with bf16 casts, which by itself sits up to ~1.2e-2 from the
+    fp32 oracle on rows that see few keys, tests/test_oracle_attention.py) within
+    TOL plus that oracle's own distance from the fp32 one."""
     got = orc.widen(out_bits, dt)
     ref32 = orc.attention_f32(q, k, v, n, offset, dt, batch=batch)
     ref16 = orc.widen(orc.attention_layer(q, k, v, n, offset, dt, batch=batch), dt)
@@ -60,6 +61,9 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None):
     e32 = float(np.abs(got - ref32).max())
     assert e32 <= TOL[dt], f"max-abs vs fp32 oracle {e32} > {TOL[dt]}"
     d16 = np.abs(got - ref16)
-    ok = (d16 <= TOL[dt]) | (d16 <= 2.0001 * ulp(ref16, dt))
+    if dt == DT_FLOAT16:
+        ok = (d16 <= TOL[dt]) | (d16 <= 2.0001 * ulp(ref16, dt))
+    else:
+        ok = d16 <= TOL[dt] + np.abs(ref16 - ref32) + 1e-7
     assert ok.all(), f"{np.count_nonzero(~ok)} elements off the layer-style oracle, worst {d16.max()}"
     return e32, float(d16.max())

@@ -69,7 +69,8 @@ int llmhip_flash_attn_opt_prefill(void *out, const void *q, const void *k, const
  * The reference has no batch dimension and no split-KV (decode there is
  * npu_flash_attn_gqa_layer with m = 1, src/llama2_layer_npu.cpp:866-869);
  * for batch == 1 this call returns what llmhip_flash_attn_gqa(m=1,
- * offset=n-1) returns.  num_splits <= 0 picks llmhip_flash_decode_default_splits.
+ * offset=n-1) returns.  num_splits <= 0 picks llmhip_flash_decode_default_splits;
+ * values above 256 are treated as 256.
  * workspace: device memory of at least llmhip_flash_decode_workspace_bytes()
  * bytes, owned by the caller, so that the call allocates nothing. */
 int llmhip_flash_decode_gqa(void *out, const void *q, const void *k_cache,

@@ -1,0 +1,198 @@
+#include "device_hip.hpp"
+
+#include <cmath>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+
+namespace llm_simple_amd {
+
+CPUAllocator &CPUAllocator::GetInstance() {
+  static CPUAllocator instance;
+  return instance;
+}
+void *CPUAllocator::Allocate(size_t size) { return std::malloc(size); }
+void CPUAllocator::Deallocate(void *ptr) { std::free(ptr); }
+
+GPUAllocator::GPUAllocator() : raw_alloc_(&llmhip_malloc), raw_free_(&llmhip_free) {}
+
+GPUAllocator &GPUAllocator::GetInstance() {
+  static GPUAllocator instance;
+  return instance;
+}
+void *GPUAllocator::Allocate(size_t size) { return GetInstance().AllocateImpl(size); }
+void GPUAllocator::Deallocate(void *ptr) { GetInstance().DeallocateImpl(ptr); }
+
+void GPUAllocator::SetBackend(RawAlloc a, RawFree f) {
+  ReleaseAll();
+  raw_alloc_ = a ? a : &llmhip_malloc;
+  raw_free_ = f ? f : &llmhip_free;
+}
+
+void GPUAllocator::ReleaseAll() {
+  for (auto &kv : cache_) {
+    raw_free_(kv.second);
+    owned_bytes_ -= kv.first;
+    ptr_size_.erase(kv.second);
+  }
+  cache_.clear();
+}
+
+void *GPUAllocator::AllocateImpl(size_t size) {
+  auto hit = cache_.lower_bound(size);  // smallest cached block that fits
+  if (hit != cache_.end()) {
+    void *p = hit->second;
+    cache_.erase(hit);
+    return p;
+  }
+  void *p = nullptr;
+  int rc = raw_alloc_(&p, size);
+  if (rc != LLMHIP_OK || p == nullptr) {
+    hip_last_status() = rc ? rc : LLMHIP_ERR_INVALID_ARG;
+    std::fprintf(stderr, "GPUAllocator: device allocation of %zu bytes failed: %s\n", size,
+                 llmhip_error_string(rc));
+    return nullptr;
+  }
+  owned_bytes_ += size;
+  ptr_size_[p] = size;
+  // after a miss, trim the cache while the pool owns more than the threshold
+  while (owned_bytes_ > dev_mem_max_ && !cache_.empty()) {
+    auto small = cache_.begin();
+    raw_free_(small->second);
+    owned_bytes_ -= small->first;
+    ptr_size_.erase(small->second);
+    cache_.erase(small);
+  }
+  return p;
+}
+
+void GPUAllocator::DeallocateImpl(void *ptr) {
+  if (ptr == nullptr) return;
+  auto it = ptr_size_.find(ptr);
+  if (it == ptr_size_.end()) {
+    std::fprintf(stderr, "GPUAllocator: %p was not allocated here\n", ptr);
+    return;
+  }
+  cache_.emplace(it->second, ptr);
+}
+
+Tensor::~Tensor() {
+  if (dev_type == DEV_GPU)
+    GPUAllocator::Deallocate(data_ptr);
+  else if (dev_type == DEV_CPU)
+    CPUAllocator::Deallocate(data_ptr);
+}
+
+std::shared_ptr<Tensor> Tensor::MakeCPUTensor(size_t size, DataType dtype) {
+  auto t = std::make_shared<Tensor>();
+  t->data_size = size;
+  t->data_type = dtype;
+  t->dev_type = DEV_CPU;
+  t->data_ptr = CPUAllocator::Allocate(SizeOfTensor(size, dtype));
+  return t;
+}
+
+std::shared_ptr<Tensor> Tensor::MakeGPUTensor(size_t size, DataType dtype) {
+  auto t = std::make_shared<Tensor>();
+  t->data_size = size;
+  t->data_type = dtype;
+  t->dev_type = DEV_GPU;
+  t->data_ptr = GPUAllocator::Allocate(SizeOfTensor(size, dtype));
+  return t;
+}
+
+std::shared_ptr<Tensor> Tensor::to(DeviceType to_dev) {
+  if (to_dev == dev_type) return shared_from_this();
+  const size_t bytes = SizeOfTensor(data_size, data_type);
+  if (dev_type == DEV_GPU && to_dev == DEV_CPU) {
+    auto r = MakeCPUTensor(data_size, data_type);
+    CHECK_LLMHIP(llmhip_memcpy_d2h(r->data_ptr, data_ptr, bytes));
+    return r;
+  }
+  if (dev_type == DEV_CPU && to_dev == DEV_GPU) {
+    auto r = MakeGPUTensor(data_size, data_type);
+    if (r->data_ptr) CHECK_LLMHIP(llmhip_memcpy_h2d(r->data_ptr, data_ptr, bytes));
+    return r;
+  }
+  return std::shared_ptr<Tensor>();
+}
+
+void Tensor::to_file(const char *path) {
+  std::shared_ptr<Tensor> host = (dev_type == DEV_CPU) ? shared_from_this() : to(DEV_CPU);
+  std::ofstream ofs(path, std::ios::binary);
+  ofs.write(static_cast<const char *>(host->data_ptr),
+            static_cast<std::streamsize>(SizeOfTensor(data_size, data_type)));
+}
+
+static inline float bf16_round_trip(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;  // nearest even, as src/util.cpp:33-72
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+std::shared_ptr<Tensor> MakeFreqCIS(int head_dim, int max_seq_len, float theta, DataType dt) {
+  const int freq_len = head_dim / 2;
+  auto t = Tensor::MakeCPUTensor(static_cast<size_t>(max_seq_len) * freq_len * 2, DT_FLOAT32);
+  float *tab = static_cast<float *>(t->data_ptr);
+  for (int j = 0; j < freq_len; ++j) {
+    const float inv = static_cast<float>(
+        1.0f / std::pow(static_cast<double>(theta), static_cast<double>(2 * j) / head_dim));
+    for (int pos = 0; pos < max_seq_len; ++pos) {
+      const float angle = static_cast<float>(pos) * inv;
+      float c = std::cos(angle), s = std::sin(angle);
+      if (dt == DT_BFLOAT16) {
+        c = bf16_round_trip(c);
+        s = bf16_round_trip(s);
+      }
+      tab[(static_cast<size_t>(pos) * freq_len + j) * 2] = c;
+      tab[(static_cast<size_t>(pos) * freq_len + j) * 2 + 1] = s;
+    }
+  }
+  return t;
+}
+
+bool AttentionGPUImpl::Init(int n_heads, int n_kv_heads, int head_dim, int max_seq_len,
+                            DataType dtype, bool rope_is_neox_style,
+                            std::shared_ptr<Tensor> freq_cis_gpu) {
+  if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || head_dim != 128 ||
+      max_seq_len < 1 || (dtype != DT_FLOAT16 && dtype != DT_BFLOAT16) || !freq_cis_gpu)
+    return false;
+  n_heads_ = n_heads;
+  n_kv_heads_ = n_kv_heads;
+  head_dim_ = head_dim;
+  max_seq_len_ = max_seq_len;
+  dtype_ = dtype;
+  neox_ = rope_is_neox_style;
+  freq_cis_ = freq_cis_gpu;
+  const size_t cache_elems = static_cast<size_t>(max_seq_len) * n_kv_heads * head_dim;
+  k_cache = Tensor::MakeGPUTensor(cache_elems, dtype);
+  v_cache = Tensor::MakeGPUTensor(cache_elems, dtype);
+  return k_cache->data_ptr != nullptr && v_cache->data_ptr != nullptr;
+}
+
+std::shared_ptr<Tensor> AttentionGPUImpl::Forward(std::shared_ptr<Tensor> q,
+                                                  std::shared_ptr<Tensor> k,
+                                                  std::shared_ptr<Tensor> v, InferenceCtx &ctx) {
+  const int cur_size = static_cast<int>(ctx.cur_size);
+  const int hidden = n_heads_ * head_dim_;
+  if (ctx.cur_pos > static_cast<size_t>(max_seq_len_)) return nullptr;
+  auto q_emb = Tensor::MakeGPUTensor(static_cast<size_t>(hidden) * cur_size, dtype_);
+  hip_rope_kv_append_layer(q_emb->data_ptr, k_cache->data_ptr, v_cache->data_ptr,
+                           freq_cis_->data_ptr, q->data_ptr, k->data_ptr, v->data_ptr,
+                           static_cast<int>(ctx.prev_pos), cur_size, n_heads_, n_kv_heads_,
+                           head_dim_, neox_, dtype_, ctx.gpu_stream);
+  auto out = Tensor::MakeGPUTensor(static_cast<size_t>(hidden) * cur_size, dtype_);
+  hip_flash_attn_gqa_layer(out->data_ptr, q_emb->data_ptr, k_cache->data_ptr, v_cache->data_ptr,
+                           cur_size, static_cast<int>(ctx.cur_pos), static_cast<int>(ctx.prev_pos),
+                           n_heads_ / n_kv_heads_, n_kv_heads_, head_dim_, dtype_, ctx.gpu_stream);
+  // q_emb goes back to the pool when this scope ends while the attention launch may
+  // still read it: drain the stream first, the rule the reference states at
+  // src/llama2_layer_npu.cpp:605-608.
+  CHECK_LLMHIP(llmhip_stream_sync(ctx.gpu_stream));
+  return out;
+}
+
+}  // namespace llm_simple_amd

@@ -311,15 +311,16 @@ static int decode_chunk(int n, int num_splits) {
 }
 
 int flash_decode_default_splits(int batch, int n, int kv_head_num) {
-  // enough workgroups to put ~4 on every one of the 256 CUs, but at least two
-  // steps (256 keys) of work in each split
+  // One workgroup per CU streams best (each keeps 64 KiB of loads in flight and
+  // fewer concurrent streams keep the HBM pages open): batch * kv heads * splits
+  // ~ 256, but at least one step (128 keys) of work per split.
   const long long pairs = (long long)batch * kv_head_num;
-  long long want = (1024 + pairs - 1) / pairs;
-  long long cap = n / (2 * kDecStepKeys);
+  long long want = (256 + pairs - 1) / pairs;
+  long long cap = n / kDecStepKeys;
   if (cap < 1) cap = 1;
   if (want > cap) want = cap;
   if (want < 1) want = 1;
-  if (want > 256) want = 256;
+  if (want > kMaxSplits) want = kMaxSplits;
   // drop splits that rounding the chunk up to whole steps would leave empty
   const int chunk = decode_chunk(n, (int)want);
   return (n + chunk - 1) / chunk;

@@ -15,6 +15,7 @@ using namespace llmhip;
 namespace {
 
 constexpr int kMaxDecodeCols = 16;
+constexpr int kMaxDecodeSplits = 256;
 
 inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 inline int from_hip(hipError_t e) { return e == hipSuccess ? LLMHIP_OK : (int)e; }
@@ -120,6 +121,7 @@ int llmhip_flash_decode_gqa(void *out, const void *q, const void *k_cache,
   if (head_dim != 128 || group_size > kMaxDecodeCols) return LLMHIP_ERR_UNSUPPORTED;
   if (batch > 65535 || kv_head_num > 65535) return LLMHIP_ERR_UNSUPPORTED;
   if (num_splits <= 0) num_splits = flash_decode_default_splits(batch, n, kv_head_num);
+  if (num_splits > kMaxDecodeSplits) num_splits = kMaxDecodeSplits;  // the combine kernel's limit
   const size_t need = flash_decode_workspace_bytes(batch, 1, group_size, kv_head_num, num_splits);
   if (need && (!workspace || workspace_bytes < need)) return LLMHIP_ERR_WORKSPACE;
   return from_hip(launch_flash_decode(out, q, k_cache, v_cache, workspace, batch, 1, n, n - 1,

@@ -1,0 +1,171 @@
+// Host-only checks of the device layer and of the C ABI's argument validation.
+// Needs no GPU: the allocator runs on an injected host backend and every ABI
+// call below is rejected (or reports "no device") before anything is launched.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "../../llm_simple_amd/csrc/device_hip.hpp"
+
+using namespace llm_simple_amd;
+
+static int g_fail = 0, g_allocs = 0, g_frees = 0;
+#define EXPECT(c)                                                       \
+  do {                                                                  \
+    if (!(c)) {                                                         \
+      std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #c);          \
+      ++g_fail;                                                         \
+    }                                                                   \
+  } while (0)
+
+static int host_alloc(void **p, size_t n) {
+  *p = std::malloc(n ? n : 1);
+  ++g_allocs;
+  return *p ? 0 : 2;
+}
+static int host_free(void *p) {
+  std::free(p);
+  ++g_frees;
+  return 0;
+}
+static int failing_alloc(void **p, size_t) {
+  *p = nullptr;
+  return 2;  // hipErrorOutOfMemory
+}
+
+static void test_sizes() {
+  EXPECT(SizeOfTensor(10, DT_FLOAT16) == 20);
+  EXPECT(SizeOfTensor(10, DT_BFLOAT16) == 20);
+  EXPECT(SizeOfTensor(10, DT_FLOAT32) == 40);
+  EXPECT(SizeOfTensor(3, DT_INT64) == 24);
+  EXPECT(SizeOfTensor(3, DT_UINT8) == 3);
+  EXPECT(SizeOfTensor(1, static_cast<DataType>(99)) == static_cast<size_t>(-1));
+  EXPECT(DEV_GPU == 1 && DT_FLOAT16 == 4 && DT_BFLOAT16 == 5);
+}
+
+static void test_allocator_pool() {
+  GPUAllocator &a = GPUAllocator::GetInstance();
+  a.SetBackend(host_alloc, host_free);
+  a.SetByteCap(1 << 20);
+  g_allocs = g_frees = 0;
+  void *p1 = GPUAllocator::Allocate(1000);
+  void *p2 = GPUAllocator::Allocate(4000);
+  void *p3 = GPUAllocator::Allocate(2000);
+  EXPECT(g_allocs == 3 && a.OwnedBytes() == 7000);
+  GPUAllocator::Deallocate(p2);
+  GPUAllocator::Deallocate(p1);
+  GPUAllocator::Deallocate(p3);
+  EXPECT(a.CachedBlocks() == 3 && g_frees == 0);
+  // smallest cached block that fits: 1500 -> the 2000-byte block, not the 4000-byte one
+  void *q = GPUAllocator::Allocate(1500);
+  EXPECT(q == p3 && g_allocs == 3);
+  void *q2 = GPUAllocator::Allocate(1000);
+  EXPECT(q2 == p1);
+  void *q3 = GPUAllocator::Allocate(5000);  // nothing fits: a fresh block
+  EXPECT(g_allocs == 4 && q3 != p2);
+  GPUAllocator::Deallocate(q);
+  GPUAllocator::Deallocate(q2);
+  GPUAllocator::Deallocate(q3);
+  // trim: with a 6000-byte threshold a miss frees cached blocks, smallest first,
+  // until the pool owns no more than the threshold (or the cache is empty)
+  a.SetByteCap(6000);
+  void *big = GPUAllocator::Allocate(9000);
+  EXPECT(big != nullptr && g_frees == 4 && a.CachedBlocks() == 0 && a.OwnedBytes() == 9000);
+  GPUAllocator::Deallocate(big);
+  a.ReleaseAll();
+  EXPECT(a.OwnedBytes() == 0 && g_frees == 5);
+  // exhaustion is reported, not fatal
+  a.SetBackend(failing_alloc, host_free);
+  hip_last_status() = 0;
+  EXPECT(GPUAllocator::Allocate(64) == nullptr && hip_last_status() != 0);
+  a.SetBackend(nullptr, nullptr);
+  a.SetByteCap(8ULL << 30);
+}
+
+static void test_tensor_cpu() {
+  auto t = Tensor::MakeCPUTensor(16, DT_FLOAT32);
+  EXPECT(t->dev_type == DEV_CPU && t->data_size == 16 && t->data_ptr != nullptr);
+  EXPECT(t->to(DEV_CPU).get() == t.get());
+  float *f = static_cast<float *>(t->data_ptr);
+  for (int i = 0; i < 16; ++i) f[i] = static_cast<float>(i);
+  t->to_file("/tmp/llm_simple_amd_tensor_test.bin");
+  std::vector<float> back(16);
+  FILE *fp = std::fopen("/tmp/llm_simple_amd_tensor_test.bin", "rb");
+  EXPECT(fp != nullptr);
+  if (fp) {
+    EXPECT(std::fread(back.data(), 4, 16, fp) == 16);
+    std::fclose(fp);
+    EXPECT(back[7] == 7.0f);
+  }
+}
+
+static void test_freq_cis() {
+  auto t = MakeFreqCIS(128, 64, 10000.0f, DT_FLOAT16);
+  const float *tab = static_cast<const float *>(t->data_ptr);
+  for (int j = 0; j < 64; ++j) EXPECT(tab[2 * j] == 1.0f && tab[2 * j + 1] == 0.0f);
+  double worst = 0;
+  for (int pos = 0; pos < 64; ++pos)
+    for (int j = 0; j < 64; ++j) {
+      const double ang = pos * std::pow(10000.0, -2.0 * j / 128.0);
+      worst = std::fmax(worst, std::fabs(tab[(pos * 64 + j) * 2] - std::cos(ang)));
+      worst = std::fmax(worst, std::fabs(tab[(pos * 64 + j) * 2 + 1] - std::sin(ang)));
+    }
+  EXPECT(worst < 2e-5);
+  auto b = MakeFreqCIS(128, 64, 1e6f, DT_BFLOAT16);
+  const uint32_t *bits = static_cast<const uint32_t *>(b->data_ptr);
+  for (int i = 0; i < 64 * 64 * 2; ++i) EXPECT((bits[i] & 0xFFFFu) == 0);  // bf16 values
+}
+
+static void test_abi_validation() {
+  char x[16];
+  void *p = x;
+  // rejected before any launch, with or without a device
+  EXPECT(llmhip_flash_attn(nullptr, p, p, p, 1, 1, 0, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_attn(p, p, p, p, 0, 1, 0, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_attn(p, p, p, p, 1, 0, 0, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_attn(p, p, p, p, 1, 1, -1, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_attn(p, p, p, p, 1, 1, 0, 1, 128, 6, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_attn(p, p, p, p, 1, 1, 0, 1, 64, 4, nullptr) == LLMHIP_ERR_UNSUPPORTED);
+  EXPECT(llmhip_flash_attn_gqa(p, p, p, p, 1, 1, 0, 0, 1, 128, 5, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_attn_gqa(p, p, p, p, 1, 1, 0, 2, 0, 128, 5, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_attn_opt_prefill(p, nullptr, p, p, 1, 1, 0, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_decode_gqa(p, p, p, p, nullptr, 0, 1, 8, 4, 1, 1, 128, 1, 5, nullptr) == LLMHIP_ERR_INVALID_ARG);  // stride < n
+  EXPECT(llmhip_flash_decode_gqa(p, p, p, p, nullptr, 0, 1, 8, 8, 17, 1, 128, 1, 5, nullptr) == LLMHIP_ERR_UNSUPPORTED);  // group > 16
+  EXPECT(llmhip_flash_decode_gqa(p, p, p, p, nullptr, 0, 1, 4096, 4096, 5, 8, 128, 4, 5, nullptr) == LLMHIP_ERR_WORKSPACE);
+  EXPECT(llmhip_flash_decode_workspace_bytes(1, 5, 8, 128, 1) == 0);
+  EXPECT(llmhip_flash_decode_workspace_bytes(2, 5, 8, 128, 4) == (size_t)2 * 8 * 4 * 16 * 130 * 4);
+  EXPECT(llmhip_flash_decode_default_splits(16, 32768, 8) == 2);
+  EXPECT(llmhip_flash_decode_default_splits(1, 100, 8) == 1);
+  EXPECT(llmhip_flash_decode_default_splits(0, 100, 8) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_rope(p, p, p, p, p, 0, 1, 2, 200, 0, 4, nullptr) == LLMHIP_ERR_UNSUPPORTED);  // hidden != heads*128
+  EXPECT(llmhip_rope(p, p, p, p, p, -1, 1, 2, 256, 0, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_rope_single(p, p, nullptr, 0, 1, 2, 256, 0, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_rope_kv_append(p, p, p, p, p, p, p, 0, 0, 2, 2, 128, 0, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_rope_kv_append(p, p, p, p, p, p, p, 0, 1, 2, 2, 96, 0, 4, nullptr) == LLMHIP_ERR_UNSUPPORTED);
+  EXPECT(llmhip_error_string(LLMHIP_ERR_WORKSPACE) != nullptr);
+  if (llmhip_device_count() == 0) {
+    void *d = nullptr, *s = nullptr;
+    EXPECT(llmhip_malloc(&d, 16) == LLMHIP_ERR_NO_DEVICE);
+    EXPECT(llmhip_stream_create(&s) == LLMHIP_ERR_NO_DEVICE);
+    EXPECT(llmhip_set_device(0) == LLMHIP_ERR_NO_DEVICE);
+    hip_last_status() = 0;
+    auto t = Tensor::MakeGPUTensor(8, DT_FLOAT16);
+    EXPECT(t->data_ptr == nullptr && hip_last_status() == LLMHIP_ERR_NO_DEVICE);
+    std::printf("no device visible: GPU paths report LLMHIP_ERR_NO_DEVICE\n");
+  }
+}
+
+int main() {
+  test_sizes();
+  test_allocator_pool();
+  test_tensor_cpu();
+  test_freq_cis();
+  test_abi_validation();
+  if (g_fail) {
+    std::printf("%d check(s) failed\n", g_fail);
+    return 1;
+  }
+  std::printf("device layer host checks: all passed\n");
+  return 0;
+}

@@ -1,0 +1,85 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads and exports
+every symbol include/llmhip.h declares, arguments are validated before any launch,
+and the C++ device layer (pooling allocator, Tensor, rotary table) behaves like the
+reference's (src/device.hpp, src/device_npu.cpp).  No GPU needed, no compute calls."""
+import ctypes
+import os
+import re
+import subprocess
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "llmhip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b(llmhip_\w+)\s*\(", text))
+
+
+def test_library_exports_every_declared_symbol():
+    import llm_simple_amd.ops as ops
+    declared = _header_symbols()
+    assert declared == set(ops.SYMBOLS), declared ^ set(ops.SYMBOLS)
+    handle = ctypes.CDLL(ops.LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), name
+
+
+def test_cpp_overloads_cover_reference_operator_names():
+    """hip_ops.hpp offers every attention / rope operator of prebuild/npu_ops.h:6-18, :39-47
+    under the same name with the npu_ prefix replaced."""
+    text = open(os.path.join(ROOT, "include", "hip_ops.hpp")).read()
+    for name in ("hip_flash_attn_layer", "hip_flash_attn_gqa_layer", "hip_flash_attn_opt_prefill_layer",
+                 "hip_rope_layer", "hip_rope_single_layer"):
+        assert re.search(r"inline void %s\(" % name, text), name
+
+
+def test_argument_validation_without_gpu():
+    import llm_simple_amd.ops as ops
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    lib = ops.lib
+    assert lib.llmhip_flash_attn(None, p, p, p, 1, 1, 0, 1, 128, 4, None) == -1
+    assert lib.llmhip_flash_attn(p, p, p, p, 1, 1, 0, 1, 64, 4, None) == -2
+    assert lib.llmhip_flash_attn_gqa(p, p, p, p, 1, 1, 0, 1, 1, 128, 7, None) == -1
+    assert lib.llmhip_flash_decode_gqa(p, p, p, p, None, 0, 1, 4096, 4096, 5, 8, 128, 4, 5, None) == -3
+    assert lib.llmhip_rope_single(p, p, p, 0, 1, 2, 100, 0, 4, None) == -2
+    try:
+        ops.hip_flash_attn_layer(0, p, p, p, 1, 1, 0, 1, 128, 4)
+    except ops.LlmHipError as e:
+        assert e.status == -1 and "invalid" in str(e)
+    else:
+        raise AssertionError("expected LlmHipError")
+
+
+def test_default_splits_and_workspace_size():
+    import llm_simple_amd.ops as ops
+    # about one workgroup per CU: batch * kv heads * splits ~ 256
+    assert ops.flash_decode_default_splits(16, 32768, 8) == 2
+    assert ops.flash_decode_default_splits(1, 32768, 8) == 32
+    assert ops.flash_decode_default_splits(1, 64, 8) == 1
+    s = ops.flash_decode_default_splits(1, 4096, 8)
+    assert 1 <= s <= 32
+    assert ops.flash_decode_workspace_bytes(1, 5, 8, 128, 1) == 0
+    assert ops.flash_decode_workspace_bytes(16, 5, 8, 128, 2) == 16 * 8 * 2 * 16 * (128 + 2) * 4
+
+
+def test_cpp_device_layer_host_checks():
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "test_device_host")
+    if not os.path.exists(exe):
+        subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "tests", "cpp")])
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "all passed" in r.stdout
+
+
+def test_product_never_touches_the_oracle():
+    """Nothing shipped imports, links or loads anything under oracle/."""
+    pkg = os.path.join(ROOT, "llm_simple_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".cpp", ".h")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f), errors="ignore").read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+    for f in ("llmhip.h", "hip_ops.hpp"):
+        assert "oracle" not in open(os.path.join(ROOT, "include", f)).read().lower()

@@ -176,6 +176,12 @@ def main():
     ap.add_argument("--seq", type=int, default=4096, help="prefill sequence length of the timed step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="comma list of legs: prefill,decode,rope (default all)")
+    ap.add_argument("--decode-shapes", default="16x32768,1x32768,1x4096,1x16384,16x4096,16x16384",
+                    help="comma list of BATCHxKVLEN decode cases; the first one is the headline")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy a few times (known traffic: 1 GiB read + "
+                         "1 GiB written per launch) so that FETCH_SIZE / WRITE_SIZE of a rocprofv3 --pmc run "
+                         "can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU; --gpus must be 1 "
@@ -190,6 +196,7 @@ def main():
     torch.cuda.set_device(0)
     timer = HipTimer(ops.lib)
     legs = set(args.only.split(",")) if args.only else {"prefill", "decode", "rope"}
+    legs.discard("none")
     extra = {}
 
     # ---- the timed step: prefill at the headline shape ----
@@ -209,7 +216,8 @@ def main():
 
     if "decode" in legs:
         dec = []
-        for batch, n in ((16, 32768), (1, 32768), (1, 4096), (1, 16384), (16, 4096), (16, 16384)):
+        shapes = [tuple(int(x) for x in c.split("x")) for c in args.decode_shapes.split(",") if c]
+        for batch, n in shapes:
             r = bench_decode(ops, torch, timer, batch, n, max(20, args.steps // 2), 10)
             log(f"decode B={batch} n={n} splits={r['splits']}: cold {r['ms_cold'] * 1e3:.1f} us "
                 f"{r['gbs_cold']:.0f} GB/s, hot {r['ms_hot'] * 1e3:.1f} us {r['gbs_hot']:.0f} GB/s")
@@ -221,7 +229,8 @@ def main():
         extra["roofline_decode"] = {
             "bound": "hbm", "achieved": head["gbs_cold"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
             "frac": head["gbs_cold"] / PEAK_HBM_GBS, "traffic": None,
-            "workload": "Qwen2.5-32B decode bf16 H=40 Hkv=8 n=32768 batch=16 (2 GiB of K+V per launch, cold)"}
+            "workload": f"Qwen2.5-32B decode bf16 H=40 Hkv=8 n={head['n']} batch={head['batch']} "
+                        f"({head['kv_bytes'] / 2 ** 20:.0f} MiB of K+V per launch, cold)"}
         extra["decode_all"] = [
             {"batch": r["batch"], "n": r["n"], "splits": r["splits"], "us_cold": r["ms_cold"] * 1e3,
              "gbs_cold": r["gbs_cold"], "frac_cold": r["gbs_cold"] / PEAK_HBM_GBS,
@@ -232,6 +241,15 @@ def main():
         log(f"rope+append S={args.seq}: {r['ms'] * 1e3:.1f} us {r['gbs']:.0f} GB/s")
         extra["rope_kv_append"] = {"S": r["S"], "us": r["ms"] * 1e3, "gbs": r["gbs"],
                                    "frac": r["gbs"] / PEAK_HBM_GBS}
+
+    if args.calib_copy:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        extra["calib_copy_bytes_each_way"] = src.numel() * 2
+        del src, dst
 
     cpu = None
     if not args.no_cpu:

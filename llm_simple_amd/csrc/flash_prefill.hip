@@ -15,16 +15,14 @@
 // permuted consistently on the V side), so P never touches LDS.  K and V tiles
 // of 64 keys are staged in LDS, XOR-swizzled 256-byte rows; K fragments are
 // read with ds_read_b128, V^T fragments with ds_read_b64_tr_b16.  exp2 with the
-// scale folded into one FMA; the running maximum is kept in raw score units; O
-// is rescaled only when some row's maximum moved.  Accumulation is fp32; out =
+// scale folded into one FMA; the reference maximum is kept in raw score units and
+// moves lazily, so O is rarely rescaled.  Accumulation is fp32; out =
 // O / l rounded once; l sums the ROUNDED probabilities (what P.V used).
 //
-// flash_prefill_kernel      4 waves, 128 query rows, two workgroups per CU:
-//                           used when the problem has few query tiles.
-// flash_prefill_pp_kernel   8 waves, 256 query rows, one workgroup per CU, two
-//                           groups of 4 waves running half an iteration apart
-//                           (one group's MFMA phase against the other group's
-//                           softmax phase), K/V tiles shared by all 8 waves.
+// flash_prefill_kernel<T, NW>: NW waves share the K/V tiles of 32*NW query rows.
+// NW = 8 (one workgroup per CU) once 256-row workgroups alone fill the chip, NW = 4
+// (two workgroups per CU) for smaller problems.  Tiles travel global -> LDS without
+// VGPR staging (global_load_lds_dwordx4), spread over the MFMA stream.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -32,6 +30,7 @@ namespace llmhip {
 
 constexpr int kTileN = 64;                      // keys per LDS tile
 constexpr int kTileBytes = kTileN * kRowBytes;  // 16 KiB
+constexpr float kLazyLog2 = 8.0f;                // rescale threshold, log2 units
 
 struct PrefillParams {
   const char *q;
@@ -154,8 +153,13 @@ template <typename T> struct WaveAttn {
     for (int kk = 0; kk < 8; ++kk) asm volatile("" : "+v"(qf[kk]));
   }
 
-  // S^T = K Q^T for the 64 keys of the tile at ks.
-  __device__ __forceinline__ void qk(const char *ks) {
+  struct NoHook {
+    __device__ __forceinline__ void operator()(int) const {}
+  };
+  // S^T = K Q^T for the 64 keys of the tile at ks.  hook(i) runs after MFMA i
+  // (0..15): the callers spread their global loads over the MFMA stream with it.
+  template <typename Hook = NoHook>
+  __device__ __forceinline__ void qk(const char *ks, Hook hook = Hook()) {
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) {
 #pragma unroll
@@ -169,6 +173,7 @@ template <typename T> struct WaveAttn {
         } else {
           s[kb] = E::mfma32(kf, qf[kk], s[kb]);
         }
+        hook(kk * 2 + kb);
       }
     }
   }
@@ -176,7 +181,8 @@ template <typename T> struct WaveAttn {
   // O^T += V^T P^T.  Lane (d = 32*dblk + l32, hh): element e of k-step (kb, ks2)
   // is the key 32*kb + 16*ks2 + 8*(e/4) + 4*hh + e%4 -- the key P's element e
   // carries.
-  __device__ __forceinline__ void pv(const char *vs) {
+  template <typename Hook = NoHook>
+  __device__ __forceinline__ void pv(const char *vs, Hook hook = Hook()) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -190,6 +196,7 @@ template <typename T> struct WaveAttn {
           const u32x2_t hi = lds_read_tr16(vs, v_swizzle_off(kr0 + 8, gran) + sub);
           const u32x4_t vf = {lo[0], lo[1], hi[0], hi[1]};
           o[d] = E::mfma32(vf, pf[kb][ks2], o[d]);
+          hook((kb * 2 + ks2) * 4 + d);
         }
       }
   }
@@ -214,7 +221,13 @@ template <typename T> struct WaveAttn {
 #pragma unroll
       for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kb][i]);
     mloc = pair_max(mloc);
-    const float m_new = fmaxf(m_run, mloc);
+    // m_run is the reference maximum used in the exponent, in raw score units.  It
+    // moves only when a row maximum exceeds it by more than kLazyLog2 in log2 units
+    // (probabilities then stay below 2^kLazyLog2, harmless in fp32 sums and in the
+    // 16-bit P operand); a -inf reference always moves.  O and l are rescaled only
+    // then, which after the first tiles is rare.
+    const bool move = mloc > m_run + kLazyLog2 / scale_log2e;
+    const float m_new = move ? mloc : m_run;
     const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
     const float neg_ms = -m_use * scale_log2e;
 #pragma unroll
@@ -222,8 +235,8 @@ template <typename T> struct WaveAttn {
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         s[kb][i] = fast_exp2(__builtin_fmaf(s[kb][i], scale_log2e, neg_ms));
-    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-      const float alpha = fast_exp2((m_run - m_use) * scale_log2e);
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      const float alpha = move ? fast_exp2((m_run - m_use) * scale_log2e) : 1.0f;
       l_run *= alpha;
 #pragma unroll
       for (int d = 0; d < 4; ++d)
@@ -268,65 +281,60 @@ template <typename T> struct WaveAttn {
   }
 };
 
-// Cooperative K or V tile loader for NT threads: thread -> row t/16 (+ NT/16 per
-// index i), 16-byte granule t%16.  The per-thread byte offset is loop invariant
-// and the tile base is wave uniform, so a full tile costs no address arithmetic;
-// only the tile that straddles row n clamps its keys.
-template <int NT> struct TileLoader {
-  static constexpr int kPer = 1024 / NT;  // granules per thread per tile
-  static constexpr int kRowStep = NT / 16;
-  int row, gi, n;
-  uint32_t off;
+// Global -> LDS tile loader without VGPR staging (global_load_lds_dwordx4: lane l's 16
+// bytes land at the wave-uniform LDS address + 16*l).  One wave instruction fills four
+// 256-byte rows; the XOR swizzles are realised on the global side: the lane that owns
+// physical granule pg of row r fetches the logical granule that belongs there.  A tile
+// is 16 instructions, dealt to the NW waves; `slot` s of wave w covers rows
+// 4*(s*NW + w) .. +3.  Completion needs s_waitcnt vmcnt(0) before the publishing barrier.
+template <int NW> struct DirectLoader {
+  static constexpr int kSlots = 16 / NW;  // instructions per wave per tile
+  int wave, lane, n;
   size_t kv_row_bytes;
-  __device__ __forceinline__ void init(int t, size_t kv_row_bytes_, int n_) {
-    row = t >> 4;
-    gi = t & 15;
+  __device__ __forceinline__ void init(int wave_, int lane_, size_t kv_row_bytes_, int n_) {
+    wave = wave_;
+    lane = lane_;
     n = n_;
     kv_row_bytes = kv_row_bytes_;
-    off = (uint32_t)row * (uint32_t)kv_row_bytes_ + (uint32_t)gi * 16u;
   }
-  __device__ __forceinline__ void load(const char *base, int t, u32x4_t (&r)[kPer]) const {
-    if ((t + 1) * kTileN <= n) {
-      const char *b_ = base + (size_t)t * kTileN * kv_row_bytes;
-#pragma unroll
-      for (int i = 0; i < kPer; ++i)
-        r[i] = global_load_b128(b_ + (size_t)i * kRowStep * kv_row_bytes + off);
-    } else {
-#pragma unroll
-      for (int i = 0; i < kPer; ++i) {
-        const int key = min(t * kTileN + row + kRowStep * i, n - 1);
-        r[i] = global_load_b128(base + (size_t)key * kv_row_bytes + gi * 16);
-      }
-    }
+  template <bool IS_V>
+  __device__ __forceinline__ void issue(const char *base, int t, char *stage, int slot) const {
+    const int r0 = 4 * (slot * NW + wave);
+    const int r = r0 + (lane >> 4), pg = lane & 15;
+    const int lg = IS_V ? ((((pg >> 2) ^ (r & 3)) << 2) | (pg & 3)) : (pg ^ (r & 15));
+    const int key = min(t * kTileN + r, n - 1);
+    const char *g = base + (size_t)key * kv_row_bytes + lg * 16;
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void *)(g),
+        (__attribute__((address_space(3))) void *)(stage + r0 * kRowBytes), 16, 0, 0);
   }
-  __device__ __forceinline__ void store_k(char *stage, const u32x4_t (&r)[kPer]) const {
-#pragma unroll
-    for (int i = 0; i < kPer; ++i)
-      lds_write_b128(stage, k_swizzle_off(row + kRowStep * i, gi), r[i]);
+  __device__ __forceinline__ void issue_k(const char *base, int t, char *stage, int slot) const {
+    issue<false>(base, t, stage, slot);
   }
-  __device__ __forceinline__ void store_v(char *stage, const u32x4_t (&r)[kPer]) const {
-#pragma unroll
-    for (int i = 0; i < kPer; ++i)
-      lds_write_b128(stage, v_swizzle_off(row + kRowStep * i, gi), r[i]);
+  __device__ __forceinline__ void issue_v(const char *base, int t, char *stage, int slot) const {
+    issue<true>(base, t, stage, slot);
   }
+  static __device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 };
 
 // ---------------------------------------------------------------------------
-// 4 waves, 128 query rows, double-buffered K/V tiles, two workgroups per CU.
+// NW waves, 32*NW query rows, double-buffered K/V tiles, one barrier per tile.
+// Every wave runs S = K Q^T, softmax and P.V of a tile as one instruction stream
+// (the compiler interleaves the softmax VALU work with the MFMAs); the loads of
+// the next tile are spread over that stream.  NW = 4: two workgroups per CU
+// (small problems); NW = 8: one workgroup per CU, K/V tiles shared by 256 rows.
 // ---------------------------------------------------------------------------
-constexpr int kSmallThreads = 256;
-constexpr int kSmallBM = 128;
-
-template <typename T>
-__global__ __launch_bounds__(kSmallThreads, 2) void flash_prefill_kernel(PrefillParams p) {
+template <typename T, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel(PrefillParams p) {
+  constexpr int BM = 32 * NW, PER = 16 / NW;  // PER: tile-load instructions per wave
   extern __shared__ __attribute__((aligned(16))) char lds[];  // [2 stages][K tile | V tile]
   int tile, head;
   if (!prefill_schedule(p, blockIdx.x, tile, head)) return;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int kvh = head / p.g;
-  const int row0 = tile * kSmallBM;
-  const int rows_end = min(p.m, row0 + kSmallBM);
+  const int row0 = tile * BM;
+  const int rows_end = min(p.m, row0 + BM);
   const int n_vis = min(p.n, rows_end + p.offset);  // keys any row of this tile can see
   const int J = (n_vis + kTileN - 1) / kTileN;
   const size_t q_row_bytes = (size_t)p.H * kRowBytes;
@@ -342,14 +350,15 @@ __global__ __launch_bounds__(kSmallThreads, 2) void flash_prefill_kernel(Prefill
   const int Jw = (qblk0 < p.m) ? min(J, (min(p.n, last_row + p.offset + 1) + kTileN - 1) / kTileN) : 0;
   w.load_q(p.q + (size_t)min(qrow, p.m - 1) * q_row_bytes + (size_t)head * kRowBytes);
 
-  TileLoader<kSmallThreads> ld;
-  ld.init(tid, kv_row_bytes, p.n);
-  u32x4_t kreg[4], vreg[4];
-  ld.load(kbase, 0, kreg);
-  ld.load(vbase, 0, vreg);
-  ld.store_k(lds, kreg);
-  ld.store_v(lds + kTileBytes, vreg);
-  w.pin_q();
+  DirectLoader<NW> ld;
+  ld.init(wave, lane, kv_row_bytes, p.n);
+#pragma unroll
+  for (int sl = 0; sl < PER; ++sl) {
+    ld.issue_k(kbase, 0, lds, sl);
+    ld.issue_v(vbase, 0, lds + kTileBytes, sl);
+  }
+  w.pin_q();  // waits for every load issued so far, the tile loads included
+  ld.wait_all();
   lds_barrier();
 
   for (int j = 0; j < J; ++j) {
@@ -357,116 +366,40 @@ __global__ __launch_bounds__(kSmallThreads, 2) void flash_prefill_kernel(Prefill
     char *vs = ks + kTileBytes;
     char *ks_next = lds + ((j + 1) & 1) * 2 * kTileBytes;
     const int jn = min(j + 1, J - 1);  // the last prefetch is redundant but branch free
-    ld.load(kbase, jn, kreg);
-    ld.load(vbase, jn, vreg);
     if (j < Jw) {
       const int key0 = j * kTileN;
       const bool partial = (key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n);
-      w.qk(ks);
+      // a burst of loads would stall every wave behind the texture addresser's queue:
+      // one load every 16 / PER MFMAs instead
+      w.qk(ks, [&](int i) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r)
+          if (i == (16 / PER) * r + 1) ld.issue_k(kbase, jn, ks_next, r);
+      });
       w.softmax(key0, qrow, p.offset, p.n, partial, p.scale_log2e);
-      w.pv(vs);
+      w.pv(vs, [&](int i) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r)
+          if (i == (16 / PER) * r + 1) ld.issue_v(vbase, jn, ks_next + kTileBytes, r);
+      });
+    } else {
+#pragma unroll
+      for (int sl = 0; sl < PER; ++sl) {
+        ld.issue_k(kbase, jn, ks_next, sl);
+        ld.issue_v(vbase, jn, ks_next + kTileBytes, sl);
+      }
     }
-    ld.store_k(ks_next, kreg);
-    ld.store_v(ks_next + kTileBytes, vreg);
+    ld.wait_all();
     lds_barrier();
   }
   w.store(p.out + (size_t)qrow * q_row_bytes + (size_t)head * kRowBytes, qrow < p.m);
 }
 
-// ---------------------------------------------------------------------------
-// 8 waves, 256 query rows, two groups of 4 waves half an iteration apart.
-//
-// Phases are separated by workgroup barriers and numbered globally: group 0
-// runs its MFMA work for tile `it` (P.V of tile it-1, then S = K Q^T of tile it)
-// in phase 2it and the softmax of tile it in phase 2it+1; group 1 does the same
-// one phase later, so each phase pairs one group's MFMAs with the other group's
-// VALU work.  K(t) is read in phases 2t and 2t+1, V(t) in phases 2t+2 and 2t+3,
-// each from a two-stage ring.  Group 0 loads K(it+1) at the start of phase 2it
-// and stores it to LDS at the end of phase 2it+1 (first read in 2it+2); group 1
-// loads V(it+1) at the start of phase 2it+2 and stores it at the end of phase
-// 2it+3 (first read in 2it+4).  Both overwrite a stage whose last reader
-// finished two barriers earlier.
-// ---------------------------------------------------------------------------
-constexpr int kPPThreads = 512;
-constexpr int kPPBM = 256;
-
-template <typename T>
-__global__ __launch_bounds__(kPPThreads, 1) void flash_prefill_pp_kernel(PrefillParams p) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];  // K0 | K1 | V0 | V1
-  int tile, head;
-  if (!prefill_schedule(p, blockIdx.x, tile, head)) return;
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int grp = wave >> 2;
-  const int kvh = head / p.g;
-  const int row0 = tile * kPPBM;
-  const int rows_end = min(p.m, row0 + kPPBM);
-  const int n_vis = min(p.n, rows_end + p.offset);
-  const int J = (n_vis + kTileN - 1) / kTileN;  // >= 1
-  const size_t q_row_bytes = (size_t)p.H * kRowBytes;
-  const size_t kv_row_bytes = (size_t)p.Hkv * kRowBytes;
-  const char *kbase = p.k + (size_t)kvh * kRowBytes;
-  const char *vbase = p.v + (size_t)kvh * kRowBytes;
-  char *const kst = lds;
-  char *const vst = lds + 2 * kTileBytes;
-
-  WaveAttn<T> w;
-  w.init(lane);
-  // query block (wave&3)*2 + grp: both groups see the same mix of diagonal work
-  const int qblk0 = row0 + ((wave & 3) * 2 + grp) * 32;
-  const int qrow = qblk0 + w.l32;
-  const int last_row = min(qblk0 + 31, p.m - 1);
-  const int Jw = (qblk0 < p.m) ? min(J, (min(p.n, last_row + p.offset + 1) + kTileN - 1) / kTileN) : 0;
-  w.load_q(p.q + (size_t)min(qrow, p.m - 1) * q_row_bytes + (size_t)head * kRowBytes);
-
-  TileLoader<256> ld;  // one group loads a whole tile
-  ld.init(tid & 255, kv_row_bytes, p.n);
-  u32x4_t rr[4];
-  {  // prologue: K(0), V(0) by group 0; K(1) by group 1
-    u32x4_t r2[4];
-    if (grp == 0) {
-      ld.load(kbase, 0, rr);
-      ld.load(vbase, 0, r2);
-      ld.store_k(kst, rr);
-      ld.store_v(vst, r2);
-    } else if (J > 1) {
-      ld.load(kbase, 1, rr);
-      ld.store_k(kst + kTileBytes, rr);
-    }
-  }
-  w.pin_q();
-  lds_barrier();
-
-  if (grp == 1) lds_barrier();
-  for (int it = 0; it <= J; ++it) {
-    // ---- MFMA phase ----
-    if (grp == 0 && it >= 1 && it + 1 < J) ld.load(kbase, it + 1, rr);
-    __builtin_amdgcn_s_setprio(2);
-    if (it >= 1 && it - 1 < Jw) w.pv(vst + ((it - 1) & 1) * kTileBytes);
-    if (it < Jw) w.qk(kst + (it & 1) * kTileBytes);
-    __builtin_amdgcn_s_setprio(0);
-    if (grp == 1 && it >= 1 && it < J) ld.store_v(vst + (it & 1) * kTileBytes, rr);
-    lds_barrier();
-    // ---- softmax phase ----
-    if (grp == 1 && it + 1 < J) ld.load(vbase, it + 1, rr);
-    if (it < Jw) {
-      const int key0 = it * kTileN;
-      const bool partial = (key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n);
-      w.softmax(key0, qrow, p.offset, p.n, partial, p.scale_log2e);
-    }
-    if (grp == 0 && it >= 1 && it + 1 < J) ld.store_k(kst + ((it + 1) & 1) * kTileBytes, rr);
-    lds_barrier();
-  }
-  if (grp == 0) lds_barrier();
-
-  w.store(p.out + (size_t)qrow * q_row_bytes + (size_t)head * kRowBytes, qrow < p.m);
-}
-
-template <typename T, bool PP>
+template <typename T, int NW>
 static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) {
   PrefillParams p = p0;
-  constexpr int BM = PP ? kPPBM : kSmallBM;
-  constexpr int NT = PP ? kPPThreads : kSmallThreads;
+  constexpr int BM = 32 * NW;
+  constexpr int NT = 64 * NW;
   p.num_q_tiles = (p.m + BM - 1) / BM;
   const int T_ = p.num_q_tiles;
   int grid;
@@ -485,7 +418,7 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
     grid = T_ * p.H;
   }
   const size_t lds_bytes = 4 * kTileBytes;
-  void (*kern)(PrefillParams) = PP ? flash_prefill_pp_kernel<T> : flash_prefill_kernel<T>;
+  void (*kern)(PrefillParams) = flash_prefill_kernel<T, NW>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -515,10 +448,10 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
   // 256-row workgroups once they alone fill the 256 CUs; 128-row ones (two per
   // CU) for smaller problems.
-  const bool pp = (long long)((m + kPPBM - 1) / kPPBM) * p.H >= 256;
+  const bool big = (long long)((m + 255) / 256) * p.H >= 256;
   if (dt == kDtFloat16)
-    return pp ? launch_prefill_t<_Float16, true>(p, stream) : launch_prefill_t<_Float16, false>(p, stream);
-  return pp ? launch_prefill_t<__bf16, true>(p, stream) : launch_prefill_t<__bf16, false>(p, stream);
+    return big ? launch_prefill_t<_Float16, 8>(p, stream) : launch_prefill_t<_Float16, 4>(p, stream);
+  return big ? launch_prefill_t<__bf16, 8>(p, stream) : launch_prefill_t<__bf16, 4>(p, stream);
 }
 
 }  // namespace llmhip

@@ -184,3 +184,77 @@ def test_qwen7b_prefill_full_size_sampled(S, rows_per_probe):
         worst = max(worst, err)
         assert err <= TOL[dt], f"row {r}: {err}"
     assert np.isfinite(orc.widen(out, dt)).all()
+
+
+def test_qwen15b_config_prefill_then_256_decode_steps():
+    """BASELINE config 3: Qwen2.5-1.5B, H=12, Hkv=2, bf16, theta 1e6 (table rounded to bf16,
+    src/model_base.cpp:59-66), neox RoPE, QKV bias ~ N(0, 0.02) in fp32 added before the single
+    rounding to bf16 (the projection epilogue, tests/gemm_test.cpp:138-149); prefill of 256 tokens,
+    then 256 decode steps with the KV cache growing in place 256 -> 512.  Every step runs the fused
+    rope + append and the attention entry point; every step is checked against the oracle."""
+    ops = _ops()
+    dt, H, Hkv, max_seq = DT_BFLOAT16, 12, 2, 512
+    rng = np.random.default_rng(1003)
+    table = orc.init_freq_cis(128, max_seq, 1e6, dt)
+    d_table = f32_dev(table)
+    bias = {name: (rng.standard_normal(h * 128, dtype=np.float32) * np.float32(0.02)) for name, h in
+            (("q", H), ("k", Hkv), ("v", Hkv))}
+
+    def projected(m, heads, name):
+        pre = orc.widen(orc.round_to(rng.standard_normal((m, heads * 128), dtype=np.float32), dt), dt)
+        return orc.round_to(pre + bias[name][None, :], dt).reshape(m, heads, 128)
+
+    kc = np.zeros((max_seq, Hkv, 128), dtype=np.uint16)
+    vc = np.zeros_like(kc)
+    d_kc, d_vc = to_dev(kc), to_dev(vc)
+    prev, worst = 0, 0.0
+    for step in range(257):
+        m = 256 if step == 0 else 1
+        cur = prev + m
+        q, k, v = projected(m, H, "q"), projected(m, Hkv, "k"), projected(m, Hkv, "v")
+        d_q, d_o = dev_empty((m, H, 128)), dev_empty((m, H, 128))
+        ops.hip_rope_kv_append_layer(d_q, d_kc, d_vc, d_table, to_dev(q), to_dev(k), to_dev(v), prev, m, H,
+                                     Hkv, 128, True, dt)
+        ops.hip_flash_attn_gqa_layer(d_o, d_q, d_kc, d_vc, m, cur, prev, H // Hkv, Hkv, 128, dt)
+        q_r = orc.rope(q, table, prev, True, dt)
+        orc.kv_append(kc, orc.rope(k, table, prev, True, dt), prev)
+        orc.kv_append(vc, v, prev)
+        ref = orc.attention_f32(q_r, kc, vc, cur, prev, dt)
+        err = float(np.abs(orc.widen(to_host(d_o), dt) - ref).max())
+        worst = max(worst, err)
+        assert err <= TOL[dt], f"step {step}: {err}"
+        prev = cur
+    assert prev == 512
+    assert np.array_equal(to_host(d_kc), kc) and np.array_equal(to_host(d_vc), vc)
+
+
+@pytest.mark.parametrize("batch,n", [(1, 32768), (16, 4096)])
+def test_qwen32b_decode_full_size(batch, n):
+    """BASELINE config 5 shape (H=40, Hkv=8, bf16) at full KV length: the CPU oracle streams the
+    same caches (decode is cheap on the CPU); plus two size-independent properties: a joint
+    permutation of the (K, V) rows leaves the output unchanged up to rounding, and the result
+    does not depend on the split count."""
+    import torch
+    ops = _ops()
+    dt, H, Hkv = DT_BFLOAT16, 40, 8
+    q = normal_bits(1005, (batch, 1, H, 128), dt)
+    k = normal_bits(1006, (batch, n, Hkv, 128), dt)
+    v = normal_bits(1007, (batch, n, Hkv, 128), dt)
+    g = H // Hkv
+
+    def run(kk, vv, splits):
+        ns = splits if splits > 0 else ops.flash_decode_default_splits(batch, n, Hkv)
+        wsb = ops.flash_decode_workspace_bytes(batch, g, Hkv, 128, ns)
+        ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
+        d_out = dev_empty((batch, 1, H, 128))
+        ops.hip_flash_decode_gqa_layer(d_out, to_dev(q), to_dev(kk), to_dev(vv), ws, wsb, batch, n, n, g, Hkv,
+                                       128, splits, dt)
+        return to_host(d_out)
+
+    out = run(k, v, 0)
+    check_attention(out, q, k, v, n, n - 1, dt, batch=True)
+    perm = np.random.default_rng(9).permutation(n)
+    out_p = run(np.ascontiguousarray(k[:, perm]), np.ascontiguousarray(v[:, perm]), 0)
+    assert np.abs(orc.widen(out, dt) - orc.widen(out_p, dt)).max() <= 2 * 2.0 ** -8
+    out_s = run(k, v, 7)
+    assert np.abs(orc.widen(out, dt) - orc.widen(out_s, dt)).max() <= 2 * 2.0 ** -8

@@ -326,8 +326,11 @@ template <int NW> struct DirectLoader {
 // ---------------------------------------------------------------------------
 template <typename T, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel(PrefillParams p) {
-  constexpr int BM = 32 * NW, PER = 16 / NW;  // PER: tile-load instructions per wave
-  extern __shared__ __attribute__((aligned(16))) char lds[];  // [2 stages][K tile | V tile]
+  // SUB tiles of 64 keys per LDS stage and per barrier: with one workgroup per CU (NW = 8)
+  // a stage holds 128 keys, which halves the number of times the waves are forced in step.
+  constexpr int BM = 32 * NW, PER = 16 / NW, SUB = NW == 8 ? 2 : 1;
+  constexpr int kStage = SUB * 2 * kTileBytes;  // [SUB x K tile | SUB x V tile]
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // 2 stages
   int tile, head;
   if (!prefill_schedule(p, blockIdx.x, tile, head)) return;
 
@@ -336,7 +339,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   const int row0 = tile * BM;
   const int rows_end = min(p.m, row0 + BM);
   const int n_vis = min(p.n, rows_end + p.offset);  // keys any row of this tile can see
-  const int J = (n_vis + kTileN - 1) / kTileN;
+  const int J = (n_vis + kTileN - 1) / kTileN;      // 64-key tiles of the workgroup
+  const int JS = (J + SUB - 1) / SUB;               // stages
   const size_t q_row_bytes = (size_t)p.H * kRowBytes;
   const size_t kv_row_bytes = (size_t)p.Hkv * kRowBytes;
   const char *kbase = p.k + (size_t)kvh * kRowBytes;
@@ -350,43 +354,51 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   const int Jw = (qblk0 < p.m) ? min(J, (min(p.n, last_row + p.offset + 1) + kTileN - 1) / kTileN) : 0;
   w.load_q(p.q + (size_t)min(qrow, p.m - 1) * q_row_bytes + (size_t)head * kRowBytes);
 
+  // tile t lives in stage (t / SUB) & 1 at sub-slot t % SUB
+  auto k_tile = [&](int t) { return lds + ((t / SUB) & 1) * kStage + (t % SUB) * kTileBytes; };
+  auto v_tile = [&](int t) { return lds + ((t / SUB) & 1) * kStage + (SUB + t % SUB) * kTileBytes; };
+
   DirectLoader<NW> ld;
   ld.init(wave, lane, kv_row_bytes, p.n);
 #pragma unroll
-  for (int sl = 0; sl < PER; ++sl) {
-    ld.issue_k(kbase, 0, lds, sl);
-    ld.issue_v(vbase, 0, lds + kTileBytes, sl);
-  }
+  for (int u = 0; u < SUB; ++u)
+#pragma unroll
+    for (int sl = 0; sl < PER; ++sl) {
+      ld.issue_k(kbase, min(u, J - 1), k_tile(u), sl);
+      ld.issue_v(vbase, min(u, J - 1), v_tile(u), sl);
+    }
   w.pin_q();  // waits for every load issued so far, the tile loads included
   ld.wait_all();
   lds_barrier();
 
-  for (int j = 0; j < J; ++j) {
-    char *ks = lds + (j & 1) * 2 * kTileBytes;
-    char *vs = ks + kTileBytes;
-    char *ks_next = lds + ((j + 1) & 1) * 2 * kTileBytes;
-    const int jn = min(j + 1, J - 1);  // the last prefetch is redundant but branch free
-    if (j < Jw) {
-      const int key0 = j * kTileN;
-      const bool partial = (key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n);
-      // a burst of loads would stall every wave behind the texture addresser's queue:
-      // one load every 16 / PER MFMAs instead
-      w.qk(ks, [&](int i) {
+  for (int js = 0; js < JS; ++js) {
 #pragma unroll
-        for (int r = 0; r < PER; ++r)
-          if (i == (16 / PER) * r + 1) ld.issue_k(kbase, jn, ks_next, r);
-      });
-      w.softmax(key0, qrow, p.offset, p.n, partial, p.scale_log2e);
-      w.pv(vs, [&](int i) {
+    for (int u = 0; u < SUB; ++u) {
+      const int j = js * SUB + u;             // tile computed now
+      const int jn = min(j + SUB, J - 1);     // tile fetched now, into the other stage
+      char *kn = k_tile(j + SUB), *vn = v_tile(j + SUB);
+      if (j < Jw) {
+        const int key0 = j * kTileN;
+        const bool partial = (key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n);
+        // a burst of loads would stall every wave behind the texture addresser's queue:
+        // one load every 16 / PER MFMAs instead
+        w.qk(k_tile(j), [&](int i) {
 #pragma unroll
-        for (int r = 0; r < PER; ++r)
-          if (i == (16 / PER) * r + 1) ld.issue_v(vbase, jn, ks_next + kTileBytes, r);
-      });
-    } else {
+          for (int r = 0; r < PER; ++r)
+            if (i == (16 / PER) * r + 1) ld.issue_k(kbase, jn, kn, r);
+        });
+        w.softmax(key0, qrow, p.offset, p.n, partial, p.scale_log2e);
+        w.pv(v_tile(j), [&](int i) {
 #pragma unroll
-      for (int sl = 0; sl < PER; ++sl) {
-        ld.issue_k(kbase, jn, ks_next, sl);
-        ld.issue_v(vbase, jn, ks_next + kTileBytes, sl);
+          for (int r = 0; r < PER; ++r)
+            if (i == (16 / PER) * r + 1) ld.issue_v(vbase, jn, vn, r);
+        });
+      } else {
+#pragma unroll
+        for (int sl = 0; sl < PER; ++sl) {
+          ld.issue_k(kbase, jn, kn, sl);
+          ld.issue_v(vbase, jn, vn, sl);
+        }
       }
     }
     ld.wait_all();
@@ -417,7 +429,7 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
     p.sched_a = 0;
     grid = T_ * p.H;
   }
-  const size_t lds_bytes = 4 * kTileBytes;
+  const size_t lds_bytes = (NW == 8 ? 2 : 1) * 4 * kTileBytes;
   void (*kern)(PrefillParams) = flash_prefill_kernel<T, NW>;
   static bool attr_set = false;
   if (!attr_set) {

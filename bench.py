@@ -31,6 +31,16 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 DT_BF16 = 5
 
+# HBM bytes per launch read off rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, FETCH_SIZE
+# scaled by 2.000 and WRITE_SIZE by 1.000, the factors a plain 1 GiB copy gives); the commands and raw
+# figures are in profiles/.  Only the shapes that were profiled have an entry.
+MEASURED_TRAFFIC_BYTES = {
+    ("prefill", 4096): (46646 + 28672) * 1024,             # algorithmic 65536 KiB
+    ("decode", 16, 32768): (2097572 + 656) * 1024,         # algorithmic 2097152 KiB
+    ("decode", 1, 32768): (131250 + 656) * 1024,           # algorithmic 131072 KiB
+    ("rope", 4096): (40530 + 36864) * 1024,                # algorithmic 75776 KiB
+}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -228,7 +238,8 @@ def main():
         extra["decode_unit"] = "GB/s"
         extra["roofline_decode"] = {
             "bound": "hbm", "achieved": head["gbs_cold"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": head["gbs_cold"] / PEAK_HBM_GBS, "traffic": None,
+            "frac": head["gbs_cold"] / PEAK_HBM_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(("decode", head["batch"], head["n"])),
             "workload": f"Qwen2.5-32B decode bf16 H=40 Hkv=8 n={head['n']} batch={head['batch']} "
                         f"({head['kv_bytes'] / 2 ** 20:.0f} MiB of K+V per launch, cold)"}
         extra["decode_all"] = [
@@ -240,7 +251,8 @@ def main():
         r = bench_rope_append(ops, torch, timer, args.seq, max(20, args.steps // 2), 10)
         log(f"rope+append S={args.seq}: {r['ms'] * 1e3:.1f} us {r['gbs']:.0f} GB/s")
         extra["rope_kv_append"] = {"S": r["S"], "us": r["ms"] * 1e3, "gbs": r["gbs"],
-                                   "frac": r["gbs"] / PEAK_HBM_GBS}
+                                   "frac": r["gbs"] / PEAK_HBM_GBS,
+                                   "traffic": MEASURED_TRAFFIC_BYTES.get(("rope", r["S"]))}
 
     if args.calib_copy:
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()
@@ -273,7 +285,8 @@ def main():
                                f"head_dim=128, S={args.seq} (BASELINE configs[3]); decode leg: "
                                f"Qwen2.5-32B H=40 Hkv=8 n=32768 (configs[4])"},
         "roofline": {"bound": "mfma", "achieved": pre["tflops"], "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": pre["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": pre["tflops"] / PEAK_BF16_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(("prefill", args.seq)),
                      "kernel": "flash_prefill_kernel<bf16>", "us_per_launch": pre["ms_event"] * 1e3,
                      "flops_per_launch": pre["flops"]},
         "cpu_baseline": cpu,

@@ -22,7 +22,13 @@
 // flash_prefill_kernel<T, NW>: NW waves share the K/V tiles of 32*NW query rows.
 // NW = 8 (one workgroup per CU) once 256-row workgroups alone fill the chip, NW = 4
 // (two workgroups per CU) for smaller problems.  Tiles travel global -> LDS without
-// VGPR staging (global_load_lds_dwordx4), spread over the MFMA stream.
+// VGPR staging (global_load_lds_dwordx4), spread over the MFMA stream.  The loop is
+// software pipelined inside a wave: the MFMAs of S(j+1) are issued beside the softmax
+// of tile j (the first ones beside the row-maximum chain, the rest, together with the
+// MFMAs of P(j).V(j), beside the exponentials), so K is fetched one tile ahead of V.
+// Every LDS fragment address is a loop-invariant register plus an immediate, and a
+// tile load is a scalar base plus a loop-invariant lane offset: the loop spends its
+// vector ALU instructions on the softmax only.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -122,13 +128,14 @@ __device__ __forceinline__ void lds_barrier() {
 template <typename T> struct WaveAttn {
   using E = Elem<T>;
   f32x16_t o[4];       // O^T: d block x (16 d rows of this lane)
-  f32x16_t s[2];       // S^T / P^T of the current tile: key block x 16 keys
   u32x4_t pf[2][2];    // P^T packed as B operand: key block x k-step
   u32x4_t qf[8];       // Q^T fragments (B operand), loaded once
   float m_run, l_run;  // running max (raw score units) and sum of this lane's keys
   int lane, l32, hh, g16, li;
+  int k_addr[8];  // LDS byte offset of this lane's K fragment kk in tile slot 0, key block 0
+  int v_addr[4];  // same for the V^T fragment of d block d (k-step 0, low half)
 
-  __device__ __forceinline__ void init(int lane_) {
+  __device__ __forceinline__ void init(int lane_, int v_region) {
     lane = lane_;
     l32 = lane & 31;
     hh = lane >> 5;
@@ -140,6 +147,20 @@ template <typename T> struct WaveAttn {
     for (int d = 0; d < 4; ++d)
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[d][i] = 0.0f;
+    // Every other fragment address of the loop is one of these plus a compile-time constant
+    // that fits the 16-bit offset field of the LDS instructions; the empty asm keeps the
+    // compiler from recomputing them (it otherwise spends ~50 VALU instructions per tile).
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      k_addr[kk] = k_swizzle_off(l32, 2 * kk + hh);
+      asm volatile("" : "+v"(k_addr[kk]));
+    }
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const int gran = d * 4 + (g16 & 1) * 2 + ((li & 3) >> 1);
+      v_addr[d] = v_region + v_swizzle_off(4 * hh + (li >> 2), gran) + (li & 1) * 8;
+      asm volatile("" : "+v"(v_addr[d]));
+    }
   }
 
   __device__ __forceinline__ void load_q(const char *q_row_head) {
@@ -156,15 +177,16 @@ template <typename T> struct WaveAttn {
   struct NoHook {
     __device__ __forceinline__ void operator()(int) const {}
   };
-  // S^T = K Q^T for the 64 keys of the tile at ks.  hook(i) runs after MFMA i
-  // (0..15): the callers spread their global loads over the MFMA stream with it.
-  template <typename Hook = NoHook>
-  __device__ __forceinline__ void qk(const char *ks, Hook hook = Hook()) {
+  // S^T = K Q^T for the 64 keys of the K tile at byte offset `koff` of the LDS segment.
+  // The fragments of step kk+1 are requested before the MFMAs of step kk.  hook(i) runs
+  // after MFMA i (0..15): the callers spread their global loads over the MFMA stream with it.
+  template <int KK0 = 0, int KK1 = 8, typename Hook = NoHook>
+  __device__ __forceinline__ void qk(const char *lds, int koff, f32x16_t (&s)[2], Hook hook = Hook()) {
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
+    for (int kk = KK0; kk < KK1; ++kk) {
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
-        const u32x4_t kf = lds_read_b128(ks, k_swizzle_off(kb * 32 + l32, 2 * kk + hh));
+        const u32x4_t kf = lds_read_b128(lds, k_addr[kk] + koff + kb * 32 * kRowBytes);
         if (kk == 0) {
           f32x16_t z;
 #pragma unroll
@@ -178,22 +200,20 @@ template <typename T> struct WaveAttn {
     }
   }
 
-  // O^T += V^T P^T.  Lane (d = 32*dblk + l32, hh): element e of k-step (kb, ks2)
-  // is the key 32*kb + 16*ks2 + 8*(e/4) + 4*hh + e%4 -- the key P's element e
-  // carries.
+  // O^T += V^T P^T over the V tile at byte offset `voff` past the start of the V region.
+  // Lane (d = 32*dblk + l32, hh): element e of k-step (kb, ks2) is the key
+  // 32*kb + 16*ks2 + 8*(e/4) + 4*hh + e%4 -- the key P's element e carries.
   template <typename Hook = NoHook>
-  __device__ __forceinline__ void pv(const char *vs, Hook hook = Hook()) {
+  __device__ __forceinline__ void pv(const char *lds, int voff, Hook hook = Hook()) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int ks2 = 0; ks2 < 2; ++ks2) {
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          const int kr0 = kb * 32 + ks2 * 16 + 4 * hh + (li >> 2);
-          const int gran = d * 4 + (g16 & 1) * 2 + ((li & 3) >> 1);
-          const int sub = (li & 1) * 8;
-          const u32x2_t lo = lds_read_tr16(vs, v_swizzle_off(kr0, gran) + sub);
-          const u32x2_t hi = lds_read_tr16(vs, v_swizzle_off(kr0 + 8, gran) + sub);
+          const int c = voff + (kb * 32 + ks2 * 16) * kRowBytes;
+          const u32x2_t lo = lds_read_tr16(lds, v_addr[d] + c);
+          const u32x2_t hi = lds_read_tr16(lds, v_addr[d] + c + 8 * kRowBytes);
           const u32x4_t vf = {lo[0], lo[1], hi[0], hi[1]};
           o[d] = E::mfma32(vf, pf[kb][ks2], o[d]);
           hook((kb * 2 + ks2) * 4 + d);
@@ -201,49 +221,20 @@ template <typename T> struct WaveAttn {
       }
   }
 
-  // Online softmax of s -> pf.  qrow: query row of this lane's column; rows see
-  // keys <= qrow + offset; `partial` says whether any key of the tile can be
-  // masked for any row of the wave.
-  __device__ __forceinline__ void softmax(int key0, int qrow, int offset, int n, bool partial,
-                                          float scale_log2e) {
-    if (partial) {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = key0 + kb * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-          if (key > qrow + offset || key >= n) s[kb][i] = -INFINITY;
-        }
-    }
-    float mloc = -INFINITY;
+  // Causal / length mask of one tile of scores (only called for tiles that can be cut).
+  __device__ __forceinline__ void mask(f32x16_t (&s)[2], int key0, int qrow, int offset, int n) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kb][i]);
-    mloc = pair_max(mloc);
-    // m_run is the reference maximum used in the exponent, in raw score units.  It
-    // moves only when a row maximum exceeds it by more than kLazyLog2 in log2 units
-    // (probabilities then stay below 2^kLazyLog2, harmless in fp32 sums and in the
-    // 16-bit P operand); a -inf reference always moves.  O and l are rescaled only
-    // then, which after the first tiles is rare.
-    const bool move = mloc > m_run + kLazyLog2 / scale_log2e;
-    const float m_new = move ? mloc : m_run;
-    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-    const float neg_ms = -m_use * scale_log2e;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        s[kb][i] = fast_exp2(__builtin_fmaf(s[kb][i], scale_log2e, neg_ms));
-    if (__builtin_amdgcn_ballot_w64(move) != 0) {
-      const float alpha = move ? fast_exp2((m_run - m_use) * scale_log2e) : 1.0f;
-      l_run *= alpha;
-#pragma unroll
-      for (int d = 0; d < 4; ++d)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
-    }
-    m_run = m_new;
+      for (int i = 0; i < 16; ++i) {
+        const int key = key0 + kb * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+        if (key > qrow + offset || key >= n) s[kb][i] = -INFINITY;
+      }
+  }
+
+  // P = exp2(s*c + neg_ms) rounded to T and packed as the B operand; returns this lane's sum
+  // of the rounded values.
+  __device__ __forceinline__ float probabilities(const f32x16_t (&s)[2], float c, float neg_ms) {
     float ps0 = 0.0f, ps1 = 0.0f;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
@@ -252,7 +243,9 @@ template <typename T> struct WaveAttn {
         u32x4_t w;
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
-          w[e2] = E::pack2(s[kb][8 * ks2 + 2 * e2], s[kb][8 * ks2 + 2 * e2 + 1]);
+          const float e0 = fast_exp2(__builtin_fmaf(s[kb][8 * ks2 + 2 * e2], c, neg_ms));
+          const float e1 = fast_exp2(__builtin_fmaf(s[kb][8 * ks2 + 2 * e2 + 1], c, neg_ms));
+          w[e2] = E::pack2(e0, e1);
           if (e2 & 1)
             ps1 = dot2_ones<T>(w[e2], ps1);
           else
@@ -260,7 +253,36 @@ template <typename T> struct WaveAttn {
         }
         pf[kb][ks2] = w;
       }
-    l_run += ps0 + ps1;
+    return ps0 + ps1;
+  }
+
+  // First half of the online softmax of one tile of (already masked) scores: row maxima and,
+  // rarely, the move of the reference.  m_run is the reference maximum used in the exponent,
+  // in raw score units.  It moves only when a row maximum exceeds it by more than kLazyLog2
+  // in log2 units (probabilities then stay below 2^kLazyLog2, harmless in fp32 sums and in
+  // the 16-bit P operand); a -inf reference always moves.  O and l are rescaled only then,
+  // which after the first tiles is rare.  Returns the additive term of the exponent.
+  __device__ __forceinline__ float row_max(const f32x16_t (&s)[2], float scale_log2e) {
+    float m0 = -INFINITY, m1 = -INFINITY;  // two chains: half the dependent latency
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      m0 = fmaxf(m0, s[0][i]);
+      m1 = fmaxf(m1, s[1][i]);
+    }
+    const float mloc = pair_max(fmaxf(m0, m1));
+    const bool move = mloc > m_run + kLazyLog2 / scale_log2e;
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      const float m_new = move ? mloc : m_run;
+      const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float alpha = move ? fast_exp2((m_run - m_use) * scale_log2e) : 1.0f;
+      l_run *= alpha;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+      m_run = m_new;
+    }
+    return -((m_run == -INFINITY) ? 0.0f : m_run) * scale_log2e;
   }
 
   // out[qrow][head][d] = O^T / l, rounded once.
@@ -282,55 +304,73 @@ template <typename T> struct WaveAttn {
 };
 
 // Global -> LDS tile loader without VGPR staging (global_load_lds_dwordx4: lane l's 16
-// bytes land at the wave-uniform LDS address + 16*l).  One wave instruction fills four
+// bytes land at the wave-uniform LDS address in M0 + 16*l).  One wave instruction fills four
 // 256-byte rows; the XOR swizzles are realised on the global side: the lane that owns
 // physical granule pg of row r fetches the logical granule that belongs there.  A tile
 // is 16 instructions, dealt to the NW waves; `slot` s of wave w covers rows
-// 4*(s*NW + w) .. +3.  Completion needs s_waitcnt vmcnt(0) before the publishing barrier.
+// 4*(s*NW + w) .. +3.  The global address is a scalar tile base plus a per-lane 32-bit
+// offset that never changes (except in a ragged last tile, whose rows are clamped to n-1),
+// so a load costs no vector ALU work.  The loads are issued from inline asm: the compiler
+// would order every later LDS read behind a transfer it knows about (s_waitcnt vmcnt(0)).
+// Completion is waited for explicitly before the barrier that publishes a stage.
 template <int NW> struct DirectLoader {
   static constexpr int kSlots = 16 / NW;  // instructions per wave per tile
-  int wave, lane, n;
-  size_t kv_row_bytes;
-  __device__ __forceinline__ void init(int wave_, int lane_, size_t kv_row_bytes_, int n_) {
-    wave = wave_;
-    lane = lane_;
+  int n, row_bytes;
+  uint32_t lds_row0;          // LDS byte offset of row 4*wave (wave-uniform)
+  int row[kSlots];            // tile row this lane fetches in slot s
+  uint32_t lane_k[kSlots];    // logical granule byte offset within the row, K swizzle
+  uint32_t lane_v[kSlots];    // same, V swizzle
+
+  __device__ __forceinline__ void init(int wave, int lane, int row_bytes_, int n_) {
     n = n_;
-    kv_row_bytes = kv_row_bytes_;
+    row_bytes = row_bytes_;
+    lds_row0 = __builtin_amdgcn_readfirstlane(4 * wave * kRowBytes);
+#pragma unroll
+    for (int s = 0; s < kSlots; ++s) {
+      const int r = 4 * (s * NW + wave) + (lane >> 4), pg = lane & 15;
+      row[s] = r;
+      lane_k[s] = (pg ^ (r & 15)) << 4;
+      lane_v[s] = ((((pg >> 2) ^ (r & 3)) << 2) | (pg & 3)) << 4;
+      asm volatile("" : "+v"(row[s]), "+v"(lane_k[s]), "+v"(lane_v[s]));
+    }
   }
+  static __device__ __forceinline__ void dma(const char *tile_base, uint32_t lane_off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_off), "s"(tile_base), "s"(lds_addr)
+                 : "m0");
+  }
+  // t: key tile; lds_tile: LDS byte offset of the destination tile
   template <bool IS_V>
-  __device__ __forceinline__ void issue(const char *base, int t, char *stage, int slot) const {
-    const int r0 = 4 * (slot * NW + wave);
-    const int r = r0 + (lane >> 4), pg = lane & 15;
-    const int lg = IS_V ? ((((pg >> 2) ^ (r & 3)) << 2) | (pg & 3)) : (pg ^ (r & 15));
-    const int key = min(t * kTileN + r, n - 1);
-    const char *g = base + (size_t)key * kv_row_bytes + lg * 16;
-    __builtin_amdgcn_global_load_lds(
-        (const __attribute__((address_space(1))) void *)(g),
-        (__attribute__((address_space(3))) void *)(stage + r0 * kRowBytes), 16, 0, 0);
-  }
-  __device__ __forceinline__ void issue_k(const char *base, int t, char *stage, int slot) const {
-    issue<false>(base, t, stage, slot);
-  }
-  __device__ __forceinline__ void issue_v(const char *base, int t, char *stage, int slot) const {
-    issue<true>(base, t, stage, slot);
+  __device__ __forceinline__ void issue(const char *base, int t, uint32_t lds_tile, int s) const {
+    const char *tile_base = base + (size_t)t * kTileN * row_bytes;
+    const uint32_t dst = lds_tile + lds_row0 + s * NW * 4 * kRowBytes;
+    // rows past n-1 (ragged last tile) are clamped to row n-1: nothing beyond the caller's n
+    // rows is read and the stale rows hold finite values; branch-free, two VALU instructions
+    const int r = min(row[s], n - 1 - t * kTileN);
+    dma(tile_base, r * row_bytes + (IS_V ? lane_v[s] : lane_k[s]), dst);
   }
   static __device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 };
 
 // ---------------------------------------------------------------------------
-// NW waves, 32*NW query rows, double-buffered K/V tiles, one barrier per tile.
-// Every wave runs S = K Q^T, softmax and P.V of a tile as one instruction stream
-// (the compiler interleaves the softmax VALU work with the MFMAs); the loads of
-// the next tile are spread over that stream.  NW = 4: two workgroups per CU
-// (small problems); NW = 8: one workgroup per CU, K/V tiles shared by 256 rows.
+// NW waves, 32*NW query rows, two LDS stages of SUB 64-key tiles, one barrier per stage.
+// Every wave runs S(j+1) = K Q^T, the softmax of tile j and P(j).V(j) as one instruction
+// stream (the compiler interleaves the softmax VALU work with the MFMAs); the tile loads
+// are spread over that stream.  NW = 4: two workgroups per CU (small problems); NW = 8:
+// one workgroup per CU, K/V tiles shared by 256 rows.
 // ---------------------------------------------------------------------------
 template <typename T, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel(PrefillParams p) {
-  // SUB tiles of 64 keys per LDS stage and per barrier: with one workgroup per CU (NW = 8)
-  // a stage holds 128 keys, which halves the number of times the waves are forced in step.
-  constexpr int BM = 32 * NW, PER = 16 / NW, SUB = NW == 8 ? 2 : 1;
-  constexpr int kStage = SUB * 2 * kTileBytes;  // [SUB x K tile | SUB x V tile]
-  extern __shared__ __attribute__((aligned(16))) char lds[];  // 2 stages
+  // SUB tiles of 64 keys per stage and per barrier: with one workgroup per CU (NW = 8) a stage
+  // holds 128 keys, which halves the number of times the waves are forced in step.
+  // LDS: K tiles of both stages [2*SUB][16 KiB], then the V tiles likewise; tile t sits in
+  // slot t % (2*SUB) of each region, so every fragment address is a per-lane register plus a
+  // constant below 64 KiB.
+  constexpr int BM = 32 * NW, PER = 16 / NW, SUB = NW == 8 ? 2 : 1, NSLOT = 2 * SUB;
+  constexpr int kVRegion = NSLOT * kTileBytes;
+  constexpr int kSplitKK = 3;  // k-steps of S(j+1) issued beside the row-maximum chain
+  extern __shared__ __attribute__((aligned(16))) char lds[];
   int tile, head;
   if (!prefill_schedule(p, blockIdx.x, tile, head)) return;
 
@@ -340,69 +380,90 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   const int rows_end = min(p.m, row0 + BM);
   const int n_vis = min(p.n, rows_end + p.offset);  // keys any row of this tile can see
   const int J = (n_vis + kTileN - 1) / kTileN;      // 64-key tiles of the workgroup
-  const int JS = (J + SUB - 1) / SUB;               // stages
   const size_t q_row_bytes = (size_t)p.H * kRowBytes;
-  const size_t kv_row_bytes = (size_t)p.Hkv * kRowBytes;
+  const int kv_row_bytes = p.Hkv * kRowBytes;
   const char *kbase = p.k + (size_t)kvh * kRowBytes;
   const char *vbase = p.v + (size_t)kvh * kRowBytes;
 
   WaveAttn<T> w;
-  w.init(lane);
+  w.init(lane, kVRegion);
   const int qblk0 = row0 + wave * 32;
   const int qrow = qblk0 + w.l32;
   const int last_row = min(qblk0 + 31, p.m - 1);
   const int Jw = (qblk0 < p.m) ? min(J, (min(p.n, last_row + p.offset + 1) + kTileN - 1) / kTileN) : 0;
   w.load_q(p.q + (size_t)min(qrow, p.m - 1) * q_row_bytes + (size_t)head * kRowBytes);
 
-  // tile t lives in stage (t / SUB) & 1 at sub-slot t % SUB
-  auto k_tile = [&](int t) { return lds + ((t / SUB) & 1) * kStage + (t % SUB) * kTileBytes; };
-  auto v_tile = [&](int t) { return lds + ((t / SUB) & 1) * kStage + (SUB + t % SUB) * kTileBytes; };
-
   DirectLoader<NW> ld;
   ld.init(wave, lane, kv_row_bytes, p.n);
+  // K runs one tile ahead of V: S(j+1) = K(j+1) Q^T is issued together with the softmax of
+  // tile j, so K tile t is fetched SUB+1 iterations and V tile t SUB iterations before use.
 #pragma unroll
-  for (int u = 0; u < SUB; ++u)
+  for (int u = 0; u <= SUB; ++u)
 #pragma unroll
     for (int sl = 0; sl < PER; ++sl) {
-      ld.issue_k(kbase, min(u, J - 1), k_tile(u), sl);
-      ld.issue_v(vbase, min(u, J - 1), v_tile(u), sl);
+      ld.template issue<false>(kbase, min(u, J - 1), (u % NSLOT) * kTileBytes, sl);
+      if (u < SUB) ld.template issue<true>(vbase, min(u, J - 1), kVRegion + u * kTileBytes, sl);
     }
-  w.pin_q();  // waits for every load issued so far, the tile loads included
+  w.pin_q();  // the Q fragments are in registers from here on
   ld.wait_all();
   lds_barrier();
 
-  for (int js = 0; js < JS; ++js) {
+  f32x16_t sa[2], sb[2];  // scores of the current / the next tile, roles alternate
+  if (Jw > 0) w.qk(lds, 0, sa);
+
+  auto tile_step = [&](int j, int slot, f32x16_t (&s_cur)[2], f32x16_t (&s_nxt)[2]) {
+    const int kslot = (slot + SUB + 1) % NSLOT, vslot = (slot + SUB) % NSLOT;  // fetched now
+    const int jk = min(j + SUB + 1, J - 1), jv = min(j + SUB, J - 1);
+    if (j < Jw) {
+      const int key0 = j * kTileN;
+      if ((key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n))
+        w.mask(s_cur, key0, qrow, p.offset, p.n);
+      // a burst of loads would stall every wave behind the texture addresser's queue:
+      // one load every 16 / PER MFMAs instead
+      auto k_hook = [&](int i) {
 #pragma unroll
-    for (int u = 0; u < SUB; ++u) {
-      const int j = js * SUB + u;             // tile computed now
-      const int jn = min(j + SUB, J - 1);     // tile fetched now, into the other stage
-      char *kn = k_tile(j + SUB), *vn = v_tile(j + SUB);
-      if (j < Jw) {
-        const int key0 = j * kTileN;
-        const bool partial = (key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n);
-        // a burst of loads would stall every wave behind the texture addresser's queue:
-        // one load every 16 / PER MFMAs instead
-        w.qk(k_tile(j), [&](int i) {
+        for (int r = 0; r < PER; ++r)
+          if (i == (16 / PER) * r + 1) ld.template issue<false>(kbase, jk, kslot * kTileBytes, r);
+      };
+      // The MFMAs of S(j+1) overlap the softmax of tile j: the first ones run beside the row
+      // maximum chain, the rest -- and the MFMAs of P.V -- beside the exponentials.  (For the
+      // wave's last tile the result is not used: one surplus pass instead of a branch that
+      // would separate these MFMAs from the instructions they overlap with.)
+      const int koff = ((slot + 1) % NSLOT) * kTileBytes;
+      w.template qk<0, kSplitKK>(lds, koff, s_nxt, k_hook);
+      const float neg_ms = w.row_max(s_cur, p.scale_log2e);
+      w.template qk<kSplitKK, 8>(lds, koff, s_nxt, k_hook);
+      w.l_run += w.probabilities(s_cur, p.scale_log2e, neg_ms);
+      w.pv(lds, slot * kTileBytes, [&](int i) {
 #pragma unroll
-          for (int r = 0; r < PER; ++r)
-            if (i == (16 / PER) * r + 1) ld.issue_k(kbase, jn, kn, r);
-        });
-        w.softmax(key0, qrow, p.offset, p.n, partial, p.scale_log2e);
-        w.pv(v_tile(j), [&](int i) {
+        for (int r = 0; r < PER; ++r)
+          if (i == (16 / PER) * r + 1)
+            ld.template issue<true>(vbase, jv, kVRegion + vslot * kTileBytes, r);
+      });
+    } else {
 #pragma unroll
-          for (int r = 0; r < PER; ++r)
-            if (i == (16 / PER) * r + 1) ld.issue_v(vbase, jn, vn, r);
-        });
-      } else {
-#pragma unroll
-        for (int sl = 0; sl < PER; ++sl) {
-          ld.issue_k(kbase, jn, kn, sl);
-          ld.issue_v(vbase, jn, vn, sl);
-        }
+      for (int sl = 0; sl < PER; ++sl) {
+        ld.template issue<false>(kbase, jk, kslot * kTileBytes, sl);
+        ld.template issue<true>(vbase, jv, kVRegion + vslot * kTileBytes, sl);
       }
     }
-    ld.wait_all();
-    lds_barrier();
+  };
+
+  for (int jb = 0; jb < J; jb += NSLOT) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+      for (int u = 0; u < SUB; ++u) {
+        const int slot = st * SUB + u;  // compile-time after unrolling
+        if (slot % 2 == 0)
+          tile_step(jb + slot, slot, sa, sb);
+        else
+          tile_step(jb + slot, slot, sb, sa);
+      }
+      ld.wait_all();
+      lds_barrier();
+      if (st == 0 && jb + SUB >= J) break;  // workgroup-uniform: the second stage holds nothing
+    }
   }
   w.store(p.out + (size_t)qrow * q_row_bytes + (size_t)head * kRowBytes, qrow < p.m);
 }

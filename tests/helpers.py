@@ -44,7 +44,7 @@ def ulp(x, dt):
     return 2.0 ** (np.floor(np.log2(ax)) - mant)
 
 
-def check_attention(out_bits, q, k, v, n, offset, dt, batch=None):
+def check_attention(out_bits, q, k, v, n, offset, dt, batch=None, layer_style=True):
     """Compare HIP output bits with both oracles.
 
     Against the fp32 oracle (the reference's test golden): max-abs <= TOL, the
@@ -53,12 +53,21 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None):
     really has) within TOL or two representable steps; bf16 (no reference code,
     the same chain with bf16 casts, which by itself sits up to ~1.2e-2 from the
     fp32 oracle on rows that see few keys, tests/test_oracle_attention.py) within
-    TOL plus that oracle's own distance from the fp32 one."""
+    TOL plus that oracle's own distance from the fp32 one.  layer_style=False skips the second
+    comparison: for scores of magnitude ~30 the layer-style chain's rounding of the scores to
+    fp16 alone (steps of 2^-6) moves the probabilities by more than TOL."""
     got = orc.widen(out_bits, dt)
     ref32 = orc.attention_f32(q, k, v, n, offset, dt, batch=batch)
     ref16 = orc.widen(orc.attention_layer(q, k, v, n, offset, dt, batch=batch), dt)
     assert np.isfinite(got).all()
     e32 = float(np.abs(got - ref32).max())
+    if not layer_style:
+        # peaked softmax rows return single V rows of magnitude up to ~4, where the rounding of
+        # the output to the storage type alone is half a step of 2^-6 (bf16): the bound scales
+        # with the magnitude of the expected value
+        rel = float((np.abs(got - ref32) / np.maximum(1.0, np.abs(ref32))).max())
+        assert rel <= TOL[dt], f"scaled max-abs vs fp32 oracle {rel} > {TOL[dt]}"
+        return e32, None
     assert e32 <= TOL[dt], f"max-abs vs fp32 oracle {e32} > {TOL[dt]}"
     d16 = np.abs(got - ref16)
     if dt == DT_FLOAT16:

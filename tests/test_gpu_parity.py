@@ -107,6 +107,59 @@ def test_flash_attn_gqa_vs_oracle(dt, m, n, offset, H, Hkv):
     check_attention(to_host(d_out), q, k, v, n, offset, dt)
 
 
+def _random_shapes():
+    """Seeded shape sweep: every loop-exit case of the prefill kernels (1..11 key tiles per
+    workgroup, ragged tails, offsets that put the diagonal anywhere in a tile), both the
+    4-wave and the 8-wave kernel (the latter needs ceil(m/256)*H >= 256)."""
+    rng = np.random.default_rng(20240607)
+    shapes = []
+    for i in range(36):
+        big = i % 3 == 0
+        m = int(rng.integers(17, 700))
+        offset = int(rng.choice([0, 0, 1, 31, 63, 64, 65, int(rng.integers(0, 400))]))
+        Hkv = int(rng.choice([1, 2, 4, 8]))
+        g = int(rng.choice([1, 2, 5, 7]))
+        if big:
+            tiles = -(-m // 256)
+            while tiles * Hkv * g < 256:
+                Hkv *= 2
+        shapes.append((m, m + offset, offset, Hkv * g, Hkv))
+    return shapes
+
+
+@pytest.mark.parametrize("idx,shape", list(enumerate(_random_shapes())))
+def test_flash_attn_shape_sweep(idx, shape):
+    ops = _ops()
+    m, n, offset, H, Hkv = shape
+    dt = DT_BFLOAT16 if idx % 2 else DT_FLOAT16
+    q = normal_bits(7000 + idx, (m, H, 128), dt)
+    k = normal_bits(7100 + idx, (n, Hkv, 128), dt)
+    v = normal_bits(7200 + idx, (n, Hkv, 128), dt)
+    d_out = dev_empty(q.shape)
+    ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), m, n, offset, H // Hkv,
+                                 Hkv, 128, dt)
+    check_attention(to_host(d_out), q, k, v, n, offset, dt)
+
+
+@pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
+@pytest.mark.parametrize("H,Hkv", [(4, 2), (64, 8)])
+def test_flash_attn_late_large_scores(dt, H, Hkv):
+    """Scores that grow along the key axis: the reference maximum of the online softmax has to
+    move many times, late in the key loop (the rescale path of the kernels), for the 4-wave
+    (H=4) and the 8-wave (H=64, m=1024) kernel."""
+    ops = _ops()
+    m = n = 1024
+    q = orc.widen(normal_bits(811, (m, H, 128), dt), dt)
+    k = orc.widen(normal_bits(812, (n, Hkv, 128), dt), dt)
+    v = normal_bits(813, (n, Hkv, 128), dt)
+    ramp = (1.0 + 3.0 * np.arange(n, dtype=np.float32) / n)[:, None, None]
+    q = orc.round_to(np.abs(q), dt)
+    k = orc.round_to(np.abs(k) * ramp, dt)
+    d_out = dev_empty(q.shape)
+    ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), m, n, 0, H // Hkv, Hkv, 128, dt)
+    check_attention(to_host(d_out), q, k, v, n, 0, dt, layer_style=False)
+
+
 def test_llama2_prefill_config_fp16():
     """BASELINE config 1: Llama2-7B prefill, fp16, H = Hkv = 32, m = n = 256, through the
     MHA entry point and the reference's own tolerance rule

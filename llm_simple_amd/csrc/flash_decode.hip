@@ -20,7 +20,11 @@
 // flash_decode_combine_kernel folds with the log-sum-exp rule.  (Folding inside
 // the last-arriving workgroup instead was measured and rejected: the device-scope
 // release/acquire fences it needs write back and invalidate the XCD's L2 and cost
-// more than the second launch -- 91 us against 33 us at batch 1, 32768 keys.)
+// more than the second launch -- 91 us against 33 us at batch 1, 32768 keys.  Without
+// fences, with the partials written through and read back at device scope (sc1 accesses)
+// and one relaxed device-scope atomic, it is correct but still slower -- 35.9 us against
+// 33.4 us, and 15.0 us against 10.6 us at 4096 keys: the chain store-acknowledge, atomic,
+// two dependent rounds of memory-latency loads in ONE workgroup is longer than a launch.)
 #include "common.hpp"
 #include "kernels.hpp"
 

@@ -89,6 +89,21 @@ inline void hip_rope_single_layer(void *output_x_dev, void *freqs_cis_dev, void 
                                   n_heads, hidden_dim, is_neox_style ? 1 : 0, dt, stream));
 }
 
+// npu_matmul_nz_layer / npu_matmul_bias_nz_layer (prebuild/npu_ops.h:87-92) with the weight
+// as W[n][k] row-major, and npu_add_layer (prebuild/npu_ops.h:80-81).
+inline void hip_matmul_layer(void *output_dev, void *lhs_dev, void *rhs_dev, int m, int n, int k,
+                             DataType dt, gpuStream_t &stream) {
+  CHECK_LLMHIP(llmhip_matmul(output_dev, lhs_dev, rhs_dev, m, n, k, dt, stream));
+}
+inline void hip_matmul_bias_layer(void *output_dev, void *lhs_dev, void *rhs_dev, void *bias_dev,
+                                  int m, int n, int k, DataType dt, gpuStream_t &stream) {
+  CHECK_LLMHIP(llmhip_matmul_bias(output_dev, lhs_dev, rhs_dev, bias_dev, m, n, k, dt, stream));
+}
+inline void hip_add_layer(void *output_dev, void *lhs, void *rhs, int total_size, DataType dt,
+                          gpuStream_t &stream) {
+  CHECK_LLMHIP(llmhip_add(output_dev, lhs, rhs, total_size, dt, stream));
+}
+
 // rope(Q), rope(K) -> k_cache[start_pos:], V -> v_cache[start_pos:] in one launch: the
 // sequence src/llama2_layer_npu.cpp:790-798 + :830-844 performs with four calls.
 inline void hip_rope_kv_append_layer(void *output_q_dev, void *k_cache_dev, void *v_cache_dev,

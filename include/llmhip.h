@@ -142,8 +142,32 @@ int llmhip_event_sync(void *event);
 int llmhip_event_elapsed_ms(float *ms, void *start, void *stop);
 const char *llmhip_error_string(int status);
 /* Frees the split-KV scratch the reference-signature attention entry points
- * keep per stream (they take no workspace argument, npu_ops.h:10-13). */
+ * keep per stream (they take no workspace argument, npu_ops.h:10-13), and the
+ * hipBLASLt handle, plans and workspace of llmhip_matmul*. */
 int llmhip_release_internal_workspace(void);
+
+/* ---- projections around the attention block (the callers either side of the path) ---- */
+
+/* Replaces npu_matmul_nz_layer (prebuild/npu_ops.h:87-88; call site
+ * src/llama2_layer_npu.cpp:1178-1180): out[m][n] = lhs[m][k] . W^T, fp32 accumulation, one
+ * rounding to dt.  `weight` is W[n][k] row-major -- the checkpoint layout -- not the
+ * reference's Ascend "nz" repacking [n/16][k][16] (tests/gemm_test.cpp:95-101).  n and k
+ * must be multiples of 16 (src/llama2_layer_npu.cpp:1211-1218).  Runs on hipBLASLt; the first
+ * call allocates the library's handle and a 64 MiB workspace. */
+int llmhip_matmul(void *out, const void *lhs, const void *weight, int m, int n, int k, int dt,
+                  void *stream);
+
+/* Replaces npu_matmul_bias_nz_layer (prebuild/npu_ops.h:90-92; call site
+ * src/llama2_layer_npu.cpp:1174-1177): as llmhip_matmul with bias[n] in fp32 added to the
+ * fp32 accumulator before the single rounding (golden tests/gemm_test.cpp:138-149). */
+int llmhip_matmul_bias(void *out, const void *lhs, const void *weight, const void *bias_f32,
+                       int m, int n, int k, int dt, void *stream);
+
+/* Replaces npu_add_layer (prebuild/npu_ops.h:80-81; call site
+ * src/llama2_layer_npu.cpp:900-901, the residual add after o_proj):
+ * out[i] = round_dt(float(lhs[i]) + float(rhs[i])). */
+int llmhip_add(void *out, const void *lhs, const void *rhs, long long total_size, int dt,
+               void *stream);
 
 #ifdef __cplusplus
 }

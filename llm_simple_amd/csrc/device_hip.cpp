@@ -1,5 +1,7 @@
 #include "device_hip.hpp"
 
+#include <cstdio>
+
 #include <cmath>
 #include <cstdint>
 #include <cstdlib>
@@ -191,6 +193,173 @@ std::shared_ptr<Tensor> AttentionGPUImpl::Forward(std::shared_ptr<Tensor> q,
   // q_emb goes back to the pool when this scope ends while the attention launch may
   // still read it: drain the stream first, the rule the reference states at
   // src/llama2_layer_npu.cpp:605-608.
+  CHECK_LLMHIP(llmhip_stream_sync(ctx.gpu_stream));
+  return out;
+}
+
+// ---------------------------------------------------------------------------
+// profiler
+// ---------------------------------------------------------------------------
+static uint64_t steady_us() {
+  return static_cast<uint64_t>(std::chrono::duration_cast<std::chrono::microseconds>(
+                                   std::chrono::steady_clock::now().time_since_epoch())
+                                   .count());
+}
+
+static std::string json_escape(const std::string &in) {
+  std::string out;
+  out.reserve(in.size() + 2);
+  for (char ch : in) {
+    switch (ch) {
+      case '"': out += "\\\""; break;
+      case '\\': out += "\\\\"; break;
+      case '\n': out += "\\n"; break;
+      case '\t': out += "\\t"; break;
+      default:
+        if (static_cast<unsigned char>(ch) < 0x20) {
+          char buf[8];
+          snprintf(buf, sizeof(buf), "\\u%04x", ch);
+          out += buf;
+        } else {
+          out += ch;
+        }
+    }
+  }
+  return out;
+}
+
+bool AppProfiler::StartLogging(const std::string &log_path) {
+  profile_file_.open(log_path.c_str());
+  if (!profile_file_) return false;
+  profile_file_ << "[\n";
+  first_record_ = true;
+  count_ = 0;
+  start_us_count_ = steady_us();
+  return true;
+}
+
+void AppProfiler::RecordEvent(const std::string &name, const std::string &info, const char *file,
+                              int lineno, uint64_t ts_us_steady, double dur_us) {
+  if (!profile_file_.is_open()) return;
+  if (first_record_)
+    first_record_ = false;
+  else
+    profile_file_ << ",\n";
+  profile_file_ << "{\"name\":\"" << json_escape(name) << "\",\"ph\":\"X\",\"pid\":0,\"ts\":"
+                << (ts_us_steady - start_us_count_) << ",\"dur\":" << dur_us
+                << ",\"args\":{\"file\":\"" << json_escape(file ? file : "") << "\",\"lineno\":" << lineno
+                << ",\"info\":\"" << json_escape(info) << "\"}}";
+  ++count_;
+}
+
+void AppProfiler::Finish() {
+  if (!profile_file_.is_open()) return;
+  profile_file_ << "\n]\n";
+  profile_file_.close();
+}
+
+AppProfileGuard::AppProfileGuard(const char *name, const char *info, gpuStream_t stream,
+                                 AppProfiler *profiler, const char *fname, int lineno,
+                                 bool is_profiling)
+    : record_name_(name), record_info_(info), record_file_name_(fname), record_file_lineno_(lineno),
+      stream_(stream), profiler_(profiler), is_profiling_(is_profiling && profiler != nullptr) {
+  if (is_profiling_) {
+    CHECK_LLMHIP(llmhip_event_create(&event_));
+    CHECK_LLMHIP(llmhip_event_record(event_, stream_));
+    start_us_ = steady_us();
+  }
+}
+
+AppProfileGuard::~AppProfileGuard() {
+  if (!is_profiling_) return;
+  void *end_event = nullptr;
+  CHECK_LLMHIP(llmhip_event_create(&end_event));
+  CHECK_LLMHIP(llmhip_event_record(end_event, stream_));
+  CHECK_LLMHIP(llmhip_stream_sync(stream_));
+  float duration_ms = 0.0f;
+  CHECK_LLMHIP(llmhip_event_elapsed_ms(&duration_ms, event_, end_event));
+  CHECK_LLMHIP(llmhip_event_destroy(event_));
+  CHECK_LLMHIP(llmhip_event_destroy(end_event));
+  profiler_->RecordEvent(record_name_, record_info_, record_file_name_, record_file_lineno_,
+                         start_us_, static_cast<double>(duration_ms) * 1000.0);
+}
+
+// ---------------------------------------------------------------------------
+// projections and the whole attention block
+// ---------------------------------------------------------------------------
+bool MatmulLayerGPUImpl::Init(const void *host_weight, const float *host_bias, size_t n_, size_t k_,
+                              DataType dtype) {
+  if (!host_weight || n_ == 0 || k_ == 0 || n_ % 16 != 0 || k_ % 16 != 0 ||
+      (dtype != DT_FLOAT16 && dtype != DT_BFLOAT16))
+    return false;
+  n = n_;
+  k = k_;
+  dtype_ = dtype;
+  weight_ = Tensor::MakeGPUTensor(n * k, dtype);
+  if (!weight_ || !weight_->data_ptr) return false;
+  if (llmhip_memcpy_h2d(weight_->data_ptr, host_weight, n * k * SizeOfTensor(1, dtype)) != 0) return false;
+  bias_.reset();
+  if (host_bias) {
+    bias_ = Tensor::MakeGPUTensor(n, DT_FLOAT32);
+    if (!bias_ || !bias_->data_ptr) return false;
+    if (llmhip_memcpy_h2d(bias_->data_ptr, host_bias, n * sizeof(float)) != 0) return false;
+  }
+  return true;
+}
+
+std::shared_ptr<Tensor> MatmulLayerGPUImpl::Forward(std::shared_ptr<Tensor> input, InferenceCtx &ctx) {
+  const int m = static_cast<int>(ctx.cur_size);
+  auto output = Tensor::MakeGPUTensor(n * ctx.cur_size, dtype_);
+  char info[96];
+  snprintf(info, sizeof(info), "m %d n %zu k %zu", m, n, k);
+  APP_PROFILE("MatmulLayer", info, ctx.gpu_stream, ctx.profiler, ctx.is_profiling);
+  if (bias_)
+    hip_matmul_bias_layer(output->data_ptr, input->data_ptr, weight_->data_ptr, bias_->data_ptr, m,
+                          static_cast<int>(n), static_cast<int>(k), dtype_, ctx.gpu_stream);
+  else
+    hip_matmul_layer(output->data_ptr, input->data_ptr, weight_->data_ptr, m, static_cast<int>(n),
+                     static_cast<int>(k), dtype_, ctx.gpu_stream);
+  return output;
+}
+
+bool AttentionBlockGPUImpl::Init(const Weights &w, int hidden_dim, int n_heads, int n_kv_heads,
+                                 int max_seq_len, DataType dtype, bool rope_is_neox_style,
+                                 std::shared_ptr<Tensor> freq_cis_gpu) {
+  if (hidden_dim < 1 || n_heads < 1 || hidden_dim % n_heads != 0) return false;
+  const int head_dim = hidden_dim / n_heads;
+  hidden_dim_ = hidden_dim;
+  dtype_ = dtype;
+  const size_t kv_dim = static_cast<size_t>(n_kv_heads) * head_dim;
+  return attention.Init(n_heads, n_kv_heads, head_dim, max_seq_len, dtype, rope_is_neox_style,
+                        freq_cis_gpu) &&
+         q_proj.Init(w.wq, w.bq, hidden_dim, hidden_dim, dtype) &&
+         k_proj.Init(w.wk, w.bk, kv_dim, hidden_dim, dtype) &&
+         v_proj.Init(w.wv, w.bv, kv_dim, hidden_dim, dtype) &&
+         o_proj.Init(w.wo, nullptr, hidden_dim, hidden_dim, dtype);
+}
+
+std::shared_ptr<Tensor> AttentionBlockGPUImpl::Forward(std::shared_ptr<Tensor> normed,
+                                                       std::shared_ptr<Tensor> residual,
+                                                       InferenceCtx &ctx) {
+  auto q = q_proj.Forward(normed, ctx);
+  auto k = k_proj.Forward(normed, ctx);
+  auto v = v_proj.Forward(normed, ctx);
+  std::shared_ptr<Tensor> attn;
+  {
+    char info[96];
+    snprintf(info, sizeof(info), "cur_size %zu cur_pos %zu", ctx.cur_size, ctx.cur_pos);
+    APP_PROFILE("RoPE+KVAppend+FlashAttnGQA", info, ctx.gpu_stream, ctx.profiler, ctx.is_profiling);
+    attn = attention.Forward(q, k, v, ctx);
+  }
+  if (!attn) return nullptr;
+  auto proj = o_proj.Forward(attn, ctx);
+  auto out = Tensor::MakeGPUTensor(static_cast<size_t>(hidden_dim_) * ctx.cur_size, dtype_);
+  {
+    APP_PROFILE("Add", "attn output + input", ctx.gpu_stream, ctx.profiler, ctx.is_profiling);
+    hip_add_layer(out->data_ptr, residual->data_ptr, proj->data_ptr,
+                  static_cast<int>(ctx.cur_size) * hidden_dim_, dtype_, ctx.gpu_stream);
+  }
+  // temporaries return to the pool at scope exit: drain first (src/llama2_layer_npu.cpp:605-608)
   CHECK_LLMHIP(llmhip_stream_sync(ctx.gpu_stream));
   return out;
 }

@@ -3,9 +3,13 @@
 // file there).  Host-only C++: everything that touches the GPU goes through
 // the C ABI of libllmhip.so.
 #pragma once
+#include <chrono>
 #include <cstddef>
+#include <cstdint>
+#include <fstream>
 #include <map>
 #include <memory>
+#include <string>
 #include <unordered_map>
 
 #include "../../include/hip_ops.hpp"
@@ -76,6 +80,54 @@ class Tensor : public std::enable_shared_from_this<Tensor> {
   DeviceType dev_type{DEV_CPU};
 };
 
+// Chrome-trace ("chrome://tracing", Perfetto) writer of the reference's profiler
+// (src/profiling.hpp, src/profiling.cpp:11-38): a JSON array of complete events
+// {"name", "ph":"X", "pid":0, "ts" (us since StartLogging), "dur" (us, GPU time between two
+// stream events), "args":{"file","lineno","info"}}.
+class AppProfiler {
+ public:
+  bool StartLogging(const std::string &log_path);
+  void RecordEvent(const std::string &name, const std::string &info, const char *file, int lineno,
+                   uint64_t ts_us_steady, double dur_us);
+  void Finish();
+  size_t EventCount() const { return count_; }
+
+ private:
+  std::ofstream profile_file_;
+  bool first_record_{true};
+  uint64_t start_us_count_{0};
+  size_t count_{0};
+};
+
+// Scope guard (src/profiling.cpp:40-94): records a stream event at construction; at
+// destruction records a second one, drains the stream and writes one trace record whose
+// duration is the GPU time between the two events.
+class AppProfileGuard {
+ public:
+  AppProfileGuard(const char *name, const char *info, gpuStream_t stream, AppProfiler *profiler,
+                  const char *fname, int lineno, bool is_profiling);
+  ~AppProfileGuard();
+  AppProfileGuard(const AppProfileGuard &) = delete;
+  AppProfileGuard &operator=(const AppProfileGuard &) = delete;
+
+ private:
+  std::string record_name_, record_info_;
+  const char *record_file_name_;
+  int record_file_lineno_;
+  gpuStream_t stream_;
+  AppProfiler *profiler_;
+  bool is_profiling_;
+  void *event_{nullptr};
+  uint64_t start_us_{0};
+};
+
+#define LLM_AMD_CONCAT2(x, y) x##y
+#define LLM_AMD_CONCAT(x, y) LLM_AMD_CONCAT2(x, y)
+// Same argument list as the reference's macro (src/profiling.hpp:47-48).
+#define APP_PROFILE(name, info, stream, profiler, isprofiling)                                   \
+  ::llm_simple_amd::AppProfileGuard LLM_AMD_CONCAT(temp_perf_obj_, __LINE__)(                    \
+      name, info, stream, profiler, __FILE__, __LINE__, isprofiling)
+
 // Positions of one step (src/model_base.hpp:40-48): cur_size = cur_pos - prev_pos
 // query tokens, keys [0, cur_pos) valid after the append.
 struct InferenceCtx {
@@ -85,6 +137,9 @@ struct InferenceCtx {
   size_t prev_pos;
   size_t cur_size;
   gpuStream_t gpu_stream;
+  // the reference reaches these through ctx.model (src/llama2_layer_npu.cpp:1169-1171)
+  AppProfiler *profiler{nullptr};
+  bool is_profiling{false};
 };
 
 // Host rotary table [max_seq_len][head_dim/2][2] = (cos, sin), built the way
@@ -114,6 +169,46 @@ class AttentionGPUImpl {
   DataType dtype_{DT_FLOAT16};
   bool neox_{false};
   std::shared_ptr<Tensor> freq_cis_;
+};
+
+// Dense projection y = x W^T (+ bias) on the GPU: MatmulLayerNPUImpl without quantisation
+// (src/llama2_layer_npu.cpp:1158-1181).  The weight is kept as W[n][k] row-major (checkpoint
+// layout); the reference's nz repacking is an Ascend detail.  bias is fp32 [n] or null
+// (src/llama2_layer_npu.cpp:1323-1338).
+class MatmulLayerGPUImpl {
+ public:
+  // host_weight: n*k elements of dtype; host_bias: n floats or nullptr.  Blocking copies.
+  bool Init(const void *host_weight, const float *host_bias, size_t n, size_t k, DataType dtype);
+  // input [cur_size][k] on the GPU -> [cur_size][n].  Asynchronous on ctx.gpu_stream.
+  std::shared_ptr<Tensor> Forward(std::shared_ptr<Tensor> input, InferenceCtx &ctx);
+  size_t n{0}, k{0};
+
+ private:
+  DataType dtype_{DT_FLOAT16};
+  std::shared_ptr<Tensor> weight_, bias_;
+};
+
+// The whole attention block of a Qwen2 / Llama-2 layer between input_norm and post_norm
+// (src/llama2_layer_npu.cpp:760-901): q/k/v projections (bias for Qwen2), RoPE + cache
+// append, attention, o_proj, residual add.
+class AttentionBlockGPUImpl {
+ public:
+  struct Weights {  // host pointers; biases may be null (Llama-2)
+    const void *wq, *wk, *wv, *wo;
+    const float *bq, *bk, *bv;
+  };
+  bool Init(const Weights &w, int hidden_dim, int n_heads, int n_kv_heads, int max_seq_len,
+            DataType dtype, bool rope_is_neox_style, std::shared_ptr<Tensor> freq_cis_gpu);
+  // normed: output of input_norm [cur_size][hidden]; residual: the layer input.  Returns
+  // residual + o_proj(attention(...)).
+  std::shared_ptr<Tensor> Forward(std::shared_ptr<Tensor> normed, std::shared_ptr<Tensor> residual,
+                                  InferenceCtx &ctx);
+  AttentionGPUImpl attention;
+  MatmulLayerGPUImpl q_proj, k_proj, v_proj, o_proj;
+
+ private:
+  int hidden_dim_{0};
+  DataType dtype_{DT_FLOAT16};
 };
 
 }  // namespace llm_simple_amd

@@ -27,4 +27,12 @@ hipError_t launch_rope_kv_append(void *out_q, void *out_k, void *out_v, const vo
                                  int start_pos, int cur_size, int q_heads, int k_heads,
                                  int k_out_row_offset, int is_neox, int dt, hipStream_t stream);
 
+// Projection GEMM through hipBLASLt: out[m][n] = round(lhs[m][k] . weight[n][k]^T + bias), bias
+// fp32 [n] or null.  The first call creates the library handle and a 64 MiB workspace.
+hipError_t launch_matmul_bias(void *out, const void *lhs, const void *weight, const float *bias,
+                              int m, int n, int k, int dt, hipStream_t stream);
+void release_matmul_resources();
+hipError_t launch_add(void *out, const void *lhs, const void *rhs, size_t total, int dt,
+                      hipStream_t stream);
+
 }  // namespace llmhip

@@ -257,7 +257,31 @@ int llmhip_release_internal_workspace(void) {
     }
   }
   g_scratch.clear();
+  release_matmul_resources();
   return rc;
+}
+
+static int matmul_common(void *out, const void *lhs, const void *weight, const void *bias, int m,
+                         int n, int k, int dt, void *stream) {
+  if (!out || !lhs || !weight) return LLMHIP_ERR_INVALID_ARG;
+  if (m < 1 || n < 1 || k < 1 || !dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
+  if (n % 16 != 0 || k % 16 != 0) return LLMHIP_ERR_UNSUPPORTED;
+  return from_hip(launch_matmul_bias(out, lhs, weight, static_cast<const float *>(bias), m, n, k, dt,
+                                     as_stream(stream)));
+}
+int llmhip_matmul(void *out, const void *lhs, const void *weight, int m, int n, int k, int dt,
+                  void *stream) {
+  return matmul_common(out, lhs, weight, nullptr, m, n, k, dt, stream);
+}
+int llmhip_matmul_bias(void *out, const void *lhs, const void *weight, const void *bias_f32, int m,
+                       int n, int k, int dt, void *stream) {
+  if (!bias_f32) return LLMHIP_ERR_INVALID_ARG;
+  return matmul_common(out, lhs, weight, bias_f32, m, n, k, dt, stream);
+}
+int llmhip_add(void *out, const void *lhs, const void *rhs, long long total_size, int dt,
+               void *stream) {
+  if (!out || !lhs || !rhs || total_size < 0 || !dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
+  return from_hip(launch_add(out, lhs, rhs, (size_t)total_size, dt, as_stream(stream)));
 }
 
 }  // extern "C"

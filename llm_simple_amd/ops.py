@@ -31,6 +31,9 @@ SYMBOLS = {
     "llmhip_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_rope_single": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_rope_kv_append": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "llmhip_matmul": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "llmhip_matmul_bias": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "llmhip_add": (_i, [_vp, _vp, _vp, ctypes.c_longlong, _i, _vp]),
     "llmhip_device_count": (_i, []),
     "llmhip_set_device": (_i, [_i]),
     "llmhip_malloc": (_i, [ctypes.POINTER(_vp), _sz]),
@@ -131,6 +134,24 @@ def flash_decode_workspace_bytes(batch, group_size, kv_head_num, head_dim, num_s
 
 def flash_decode_default_splits(batch, n, kv_head_num):
     return lib.llmhip_flash_decode_default_splits(batch, n, kv_head_num)
+
+
+def hip_matmul_layer(output_dev, lhs_dev, weight_dev, m, n, k, dt, stream=0):
+    """npu_matmul_nz_layer (prebuild/npu_ops.h:87-88) with the weight as W[n][k] row-major."""
+    _check(lib.llmhip_matmul(_ptr(output_dev), _ptr(lhs_dev), _ptr(weight_dev), m, n, k, dt, stream),
+           "hip_matmul_layer")
+
+
+def hip_matmul_bias_layer(output_dev, lhs_dev, weight_dev, bias_dev, m, n, k, dt, stream=0):
+    """npu_matmul_bias_nz_layer (prebuild/npu_ops.h:90-92): fp32 bias added before the rounding."""
+    _check(lib.llmhip_matmul_bias(_ptr(output_dev), _ptr(lhs_dev), _ptr(weight_dev), _ptr(bias_dev),
+                                  m, n, k, dt, stream), "hip_matmul_bias_layer")
+
+
+def hip_add_layer(output_dev, lhs_dev, rhs_dev, total_size, dt, stream=0):
+    """npu_add_layer (prebuild/npu_ops.h:80-81)."""
+    _check(lib.llmhip_add(_ptr(output_dev), _ptr(lhs_dev), _ptr(rhs_dev), total_size, dt, stream),
+           "hip_add_layer")
 
 
 def hip_rope_layer(output_q_dev, output_k_dev, freqs_cis_dev, input_q_dev, input_k_dev, start_pos,

@@ -29,6 +29,11 @@
  *                          test: PARITY UNPINNED against the reference at that
  *                          point; pinned only against the HF repeat_kv
  *                          convention (repeat_interleave on K/V).
+ *   orc_matmul_bias        pinned: numpy float64 matmul + bias within one
+ *                          step of the storage type, identity weight, zero
+ *                          input (output == rounded bias), row/column
+ *                          permutation equivariance.
+ *   orc_add                pinned: numpy float32 add + the pinned rounding.
  *
  * Build: see oracle/Makefile (gcc -O3 -ffp-contract=off -fopenmp).
  * -ffp-contract=off keeps a*b-c*d as two roundings + one, exactly what the
@@ -323,6 +328,52 @@ void orc_attention_f32(float *out, const uint16_t *q, const uint16_t *k, const u
 #endif
   attention_body(NULL, out, q, k, v, batch, m, n, offset, group_size, kv_head_num,
                  head_dim, kv_seq_stride, dt, 0);
+}
+
+/* ---------------------------------------------------------------- */
+/* projections either side of the attention block                    */
+/* ---------------------------------------------------------------- */
+
+/* out[m][n] = round_T(sum_k lhs[m][k] * w[n][k] + bias[n]): the golden of
+ * tests/gemm_test.cpp:138-149 (fp32 contraction, fp32 bias broadcast over the
+ * rows, one cast to T).  w is W[n][k] row-major, i.e. the transpose of the
+ * [k][n] right-hand side the reference test builds before it repacks it into the
+ * Ascend nz layout (tests/gemm_test.cpp:88-101).  bias may be NULL
+ * (npu_matmul_nz_layer).  The order of the fp32 summation inside Eigen's
+ * contraction is not specified; eight interleaved partial sums are used. */
+void orc_matmul_bias(uint16_t *out, const uint16_t *lhs, const uint16_t *w, const float *bias,
+                     int m, int n, int k, int dt, int n_threads) {
+  float *wf = (float *)malloc((size_t)n * k * sizeof(float));
+  float *xf = (float *)malloc((size_t)m * k * sizeof(float));
+  orc_widen_array(wf, w, (int64_t)n * k, dt);
+  orc_widen_array(xf, lhs, (int64_t)m * k, dt);
+#ifdef _OPENMP
+  if (n_threads <= 0) n_threads = omp_get_max_threads();
+#pragma omp parallel for num_threads(n_threads) schedule(static)
+#endif
+  for (int i = 0; i < m; ++i) {
+    const float *x = xf + (size_t)i * k;
+    for (int j = 0; j < n; ++j) {
+      const float *wr = wf + (size_t)j * k;
+      float p[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      int c = 0;
+      for (; c + 8 <= k; c += 8)
+        for (int e = 0; e < 8; ++e) p[e] += x[c + e] * wr[c + e];
+      for (; c < k; ++c) p[c & 7] += x[c] * wr[c];
+      float acc = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+      if (bias) acc += bias[j];
+      out[(size_t)i * n + j] = round_t(acc, dt);
+    }
+  }
+  (void)n_threads;
+  free(wf);
+  free(xf);
+}
+
+/* out[i] = round_T(float(lhs[i]) + float(rhs[i])): the residual add after o_proj
+ * (npu_add_layer, src/llama2_layer_npu.cpp:900-901). */
+void orc_add(uint16_t *out, const uint16_t *lhs, const uint16_t *rhs, int64_t count, int dt) {
+  for (int64_t i = 0; i < count; ++i) out[i] = round_t(load_t(lhs + i, dt) + load_t(rhs + i, dt), dt);
 }
 
 /* Comparison rule of the reference's tests (tests/npu_op_test_util.cpp:33-48):

@@ -41,6 +41,8 @@ def _load():
     h.orc_kv_append.argtypes = [vp, vp, i, i, i]
     h.orc_attention_layer.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, i, i64, i, i]
     h.orc_attention_f32.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, i, i64, i, i]
+    h.orc_matmul_bias.argtypes = [vp, vp, vp, vp, i, i, i, i, i]
+    h.orc_add.argtypes = [vp, vp, vp, i64, i]
     h.orc_all_close.restype = i64
     h.orc_all_close.argtypes = [vp, vp, i64, f, f, ctypes.POINTER(f)]
     h.orc_max_threads.restype = i
@@ -145,6 +147,30 @@ def attention_f32(q, k, v, n, offset, dt, batch=None, n_threads=0):
     out = np.empty(q.shape, dtype=np.float32)
     _h.orc_attention_f32(_p(out), _p(q), _p(k), _p(v), b, m, n, offset, H // Hkv, Hkv, hd,
                          stride, dt, n_threads)
+    return out
+
+
+def matmul_bias(lhs_bits, w_bits, bias, dt, n_threads=0):
+    """round(lhs[m][k] . w[n][k]^T + bias[n]) -> bits [m][n]; bias fp32 or None."""
+    lhs_bits = _c(lhs_bits, np.uint16)
+    w_bits = _c(w_bits, np.uint16)
+    m, k = lhs_bits.shape
+    n, k2 = w_bits.shape
+    assert k == k2
+    out = np.empty((m, n), dtype=np.uint16)
+    b = None if bias is None else _c(bias, np.float32)
+    assert b is None or b.shape == (n,)
+    _h.orc_matmul_bias(_p(out), _p(lhs_bits), _p(w_bits), None if b is None else _p(b), m, n, k, dt,
+                       n_threads)
+    return out
+
+
+def add(lhs_bits, rhs_bits, dt):
+    lhs_bits = _c(lhs_bits, np.uint16)
+    rhs_bits = _c(rhs_bits, np.uint16)
+    assert lhs_bits.shape == rhs_bits.shape
+    out = np.empty(lhs_bits.shape, dtype=np.uint16)
+    _h.orc_add(_p(out), _p(lhs_bits), _p(rhs_bits), lhs_bits.size, dt)
     return out
 
 

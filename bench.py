@@ -153,6 +153,60 @@ def bench_rope_append(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
     return {"S": S, "ms": ms, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9}
 
 
+def bench_attention_block(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
+    """The whole attention block of one Qwen2.5-7B layer (src/llama2_layer_npu.cpp:760-901):
+    q/k/v projections with fp32 bias (hipBLASLt), fused RoPE + KV append, causal attention, o_proj,
+    residual add -- random weights of that shape, one sequence of S tokens."""
+    import numpy as np
+    hidden, kvd = H * 128, Hkv * 128
+    g = torch.Generator(device="cuda").manual_seed(11)
+    bf = torch.bfloat16
+
+    def rnd(*shape, scale=1.0):
+        return (torch.randn(*shape, device="cuda", dtype=torch.float32, generator=g) * scale).to(bf)
+
+    x, res = rnd(S, hidden), rnd(S, hidden)
+    wq, wo = rnd(hidden, hidden, scale=hidden ** -0.5), rnd(hidden, hidden, scale=hidden ** -0.5)
+    wk, wv = rnd(kvd, hidden, scale=hidden ** -0.5), rnd(kvd, hidden, scale=hidden ** -0.5)
+    bq = torch.randn(hidden, device="cuda", generator=g) * 0.02
+    bk = torch.randn(kvd, device="cuda", generator=g) * 0.02
+    bv = torch.randn(kvd, device="cuda", generator=g) * 0.02
+    q, k, v = torch.empty(S, hidden, device="cuda", dtype=bf), torch.empty(S, kvd, device="cuda", dtype=bf), \
+        torch.empty(S, kvd, device="cuda", dtype=bf)
+    qe, attn, proj, out = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    kc, vc = torch.empty(S, kvd, device="cuda", dtype=bf), torch.empty(S, kvd, device="cuda", dtype=bf)
+    table = torch.from_numpy(np.ascontiguousarray(ops.init_freq_cis(128, S, 1e6, DT_BF16))).cuda()
+
+    def proj_qkv(_):
+        ops.hip_matmul_bias_layer(q, x, wq, bq, S, hidden, hidden, DT_BF16)
+        ops.hip_matmul_bias_layer(k, x, wk, bk, S, kvd, hidden, DT_BF16)
+        ops.hip_matmul_bias_layer(v, x, wv, bv, S, kvd, hidden, DT_BF16)
+
+    def core(_):
+        ops.hip_rope_kv_append_layer(qe, kc, vc, table, q, k, v, 0, S, H, Hkv, 128, True, DT_BF16)
+        ops.hip_flash_attn_gqa_layer(attn, qe, kc, vc, S, S, 0, H // Hkv, Hkv, 128, DT_BF16)
+
+    def tail(_):
+        ops.hip_matmul_layer(proj, attn, wo, S, hidden, hidden, DT_BF16)
+        ops.hip_add_layer(out, res, proj, S * hidden, DT_BF16)
+
+    def whole(i):
+        proj_qkv(i)
+        core(i)
+        tail(i)
+
+    for i in range(warmup):
+        whole(i)
+    torch.cuda.synchronize()
+    r = {"S": S}
+    for name, fn in (("us_total", whole), ("us_qkv_proj", proj_qkv), ("us_rope_attention", core),
+                     ("us_o_proj_add", tail)):
+        r[name] = median([timer.time_ms(fn, steps) for _ in range(3)]) * 1e3
+    gemm_flops = 2.0 * S * hidden * (2 * hidden + 2 * kvd)
+    r["gemm_tflops"] = gemm_flops / ((r["us_qkv_proj"] + r["us_o_proj_add"]) * 1e-6) / 1e12
+    return r
+
+
 def cpu_baseline(S, H=28, Hkv=4):
     """The oracle's layer-style attention (the port of the reference CPU layer
     path) on the whole prefill workload: single thread (the reference's Eigen
@@ -185,7 +239,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--seq", type=int, default=4096, help="prefill sequence length of the timed step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: prefill,decode,rope (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs: prefill,decode,rope,block (default all)")
     ap.add_argument("--decode-shapes", default="16x32768,1x32768,1x4096,1x16384,16x4096,16x16384",
                     help="comma list of BATCHxKVLEN decode cases; the first one is the headline")
     ap.add_argument("--calib-copy", action="store_true",
@@ -205,7 +259,7 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     timer = HipTimer(ops.lib)
-    legs = set(args.only.split(",")) if args.only else {"prefill", "decode", "rope"}
+    legs = set(args.only.split(",")) if args.only else {"prefill", "decode", "rope", "block"}
     legs.discard("none")
     extra = {}
 
@@ -253,6 +307,13 @@ def main():
         extra["rope_kv_append"] = {"S": r["S"], "us": r["ms"] * 1e3, "gbs": r["gbs"],
                                    "frac": r["gbs"] / PEAK_HBM_GBS,
                                    "traffic": MEASURED_TRAFFIC_BYTES.get(("rope", r["S"]))}
+
+    if "block" in legs:
+        r = bench_attention_block(ops, torch, timer, args.seq, max(10, args.steps // 8), 3)
+        log(f"attention block S={args.seq}: {r['us_total']:.0f} us (qkv proj {r['us_qkv_proj']:.0f}, "
+            f"rope+attention {r['us_rope_attention']:.0f}, o_proj+add {r['us_o_proj_add']:.0f}; "
+            f"GEMMs {r['gemm_tflops']:.0f} TFLOP/s)")
+        extra["attention_block"] = r
 
     if args.calib_copy:
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()

@@ -22,6 +22,9 @@ void orc_kv_append(uint16_t *cache, const uint16_t *src, int prev_pos, int cur_s
 void orc_attention_f32(float *out, const uint16_t *q, const uint16_t *k, const uint16_t *v, int batch,
                        int m, int n, int offset, int group_size, int kv_head_num, int head_dim,
                        int64_t kv_seq_stride, int dt, int n_threads);
+void orc_matmul_bias(uint16_t *out, const uint16_t *lhs, const uint16_t *w, const float *bias, int m, int n,
+                     int k, int dt, int n_threads);
+void orc_add(uint16_t *out, const uint16_t *lhs, const uint16_t *rhs, int64_t count, int dt);
 int64_t orc_all_close(const float *a, const float *b, int64_t count, float abs_err, float rel_err,
                       float *max_abs_out);
 }
@@ -68,6 +71,22 @@ inline std::vector<uint16_t> normal_bits(uint64_t seed, size_t count, int dt) {
   std::vector<uint16_t> b(count);
   orc_round_array(b.data(), f.data(), static_cast<int64_t>(count), dt);
   return b;
+}
+
+// N(0, sigma) weights rounded to the storage type
+inline std::vector<uint16_t> scaled_normal_bits(uint64_t seed, size_t count, float sigma, int dt) {
+  Rng r(seed);
+  std::vector<float> f(count);
+  for (auto &x : f) x = sigma * r.normal();
+  std::vector<uint16_t> b(count);
+  orc_round_array(b.data(), f.data(), static_cast<int64_t>(count), dt);
+  return b;
+}
+inline std::vector<float> normal_f32(uint64_t seed, size_t count, float sigma) {
+  Rng r(seed);
+  std::vector<float> f(count);
+  for (auto &x : f) x = sigma * r.normal();
+  return f;
 }
 
 inline std::shared_ptr<llm_simple_amd::Tensor> to_gpu(const void *host, size_t elems,

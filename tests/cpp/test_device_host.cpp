@@ -2,7 +2,11 @@
 // Needs no GPU: the allocator runs on an injected host backend and every ABI
 // call below is rejected (or reports "no device") before anything is launched.
 #include <cmath>
+#include <chrono>
 #include <cstdio>
+#include <fstream>
+#include <iterator>
+#include <string>
 #include <cstdlib>
 #include <vector>
 
@@ -156,7 +160,42 @@ static void test_abi_validation() {
   }
 }
 
+// The profiler's file is a JSON array of Chrome-trace complete events
+// (src/profiling.cpp:11-38, :80-93); RecordEvent is exercised directly, the GPU-timed guard
+// belongs to the GPU tests.
+static void test_profiler_file() {
+  const char *path = "/tmp/llm_simple_amd_profiler_test.json";
+  AppProfiler prof;
+  EXPECT(prof.StartLogging(path));
+  const uint64_t now = static_cast<uint64_t>(std::chrono::duration_cast<std::chrono::microseconds>(
+                                                 std::chrono::steady_clock::now().time_since_epoch())
+                                                 .count());
+  prof.RecordEvent("MatmulLayer", "m 1 n 16 k \"16\"", "a\\b.cpp", 42, now + 5, 12.5);
+  prof.RecordEvent("Add", "attn output + input", "x.cpp", 7, now + 30, 1.0);
+  EXPECT(prof.EventCount() == 2);
+  prof.Finish();
+  std::ifstream in(path);
+  std::string text((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+  EXPECT(text.rfind("[\n", 0) == 0);
+  EXPECT(text.find("{\"name\":\"MatmulLayer\",\"ph\":\"X\",\"pid\":0,\"ts\":") != std::string::npos);
+  EXPECT(text.find("\"dur\":12.5,\"args\":{\"file\":\"a\\\\b.cpp\",\"lineno\":42,\"info\":\"m 1 n 16 k \\\"16\\\"\"}}") !=
+        std::string::npos);
+  EXPECT(text.find("},\n{\"name\":\"Add\"") != std::string::npos);
+  EXPECT(text.size() > 3 && text.substr(text.size() - 3) == "\n]\n");
+  AppProfiler closed;
+  closed.RecordEvent("x", "y", "z", 1, now, 1.0);  // not started: ignored
+  EXPECT(closed.EventCount() == 0);
+  EXPECT(!closed.StartLogging("/nonexistent-dir/trace.json"));
+  // a projection layer refuses what the kernels cannot take, before touching the device
+  MatmulLayerGPUImpl mm;
+  uint16_t dummy = 0;
+  EXPECT(!mm.Init(&dummy, nullptr, 15, 16, DT_FLOAT16));
+  EXPECT(!mm.Init(&dummy, nullptr, 16, 16, DT_FLOAT32));
+  EXPECT(!mm.Init(nullptr, nullptr, 16, 16, DT_FLOAT16));
+}
+
 int main() {
+  test_profiler_file();
   test_sizes();
   test_allocator_pool();
   test_tensor_cpu();

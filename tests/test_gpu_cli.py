@@ -14,7 +14,7 @@ BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "bin")
 def _run(exe, *flags):
     print("running", exe, *flags, flush=True)
     r = subprocess.run([os.path.join(BIN, exe), *map(str, flags)], capture_output=True, text=True, timeout=300)
-    assert r.returncode == 0 and "PASS" in r.stdout, r.stdout + r.stderr
+    assert r.returncode == 0 and ("PASS" in r.stdout or "test success" in r.stdout), r.stdout + r.stderr
     return r.stdout
 
 
@@ -46,3 +46,36 @@ def test_op_test_rope_single(flags):
 ])
 def test_attention_layer_prefill_then_decode(flags):
     _run("op_test_attention_layer", *flags)
+
+
+@pytest.mark.parametrize("flags", [
+    ("--m", 2048, "--n", 2048, "--k", 2048, "--dtype", "fp16"),                       # the reference CLI's defaults
+    ("--m", 256, "--n", 3584, "--k", 3584, "--bias", 1, "--dtype", "bf16"),           # Qwen2.5-7B q_proj
+    ("--m", 1, "--n", 512, "--k", 3584, "--bias", 1, "--dtype", "bf16"),              # k_proj, decode
+])
+def test_op_test_gemm(flags):
+    _run("op_test_gemm", *flags)
+
+
+@pytest.mark.parametrize("flags", [
+    ("--head_num", 12, "--kv_head_num", 2, "--prompt", 256, "--steps", 6, "--dtype", "bf16"),     # Qwen2.5-1.5B shape
+    ("--head_num", 28, "--kv_head_num", 4, "--prompt", 512, "--steps", 2, "--dtype", "bf16",
+     "--max_seq_len", 1024),                                                                      # Qwen2.5-7B shape
+    ("--head_num", 8, "--kv_head_num", 8, "--prompt", 40, "--steps", 3, "--dtype", "fp16", "--is_neox", 0,
+     "--theta", 10000, "--bias", 0),                                                              # Llama-style
+])
+def test_attention_block_with_projections_and_trace(flags, tmp_path):
+    """q/k/v projections -> RoPE + append -> attention -> o_proj -> residual add, profiled: the
+    trace file must be the Chrome-trace JSON the reference's profiler writes
+    (src/profiling.cpp:11-38, :80-93)."""
+    import json
+    trace = tmp_path / "trace.json"
+    _run("op_test_attention_block", *flags, "--trace", trace)
+    events = json.loads(trace.read_text())
+    steps = flags[flags.index("--steps") + 1]
+    assert len(events) == 6 * (steps + 1)
+    names = [e["name"] for e in events[:6]]
+    assert names == ["MatmulLayer"] * 3 + ["RoPE+KVAppend+FlashAttnGQA", "MatmulLayer", "Add"]
+    for e in events:
+        assert e["ph"] == "X" and e["pid"] == 0 and e["dur"] > 0 and e["ts"] >= 0
+        assert set(e["args"]) == {"file", "lineno", "info"}

@@ -285,11 +285,15 @@ template <typename T> struct WaveAttn {
     return -((m_run == -INFINITY) ? 0.0f : m_run) * scale_log2e;
   }
 
-  // out[qrow][head][d] = O^T / l, rounded once.
-  __device__ __forceinline__ void store(char *out_row_head, bool valid) {
+  // out[row][head][0..127] = O^T / l, rounded once.  The lane layout of O^T (a lane holds 4
+  // contiguous dims of one row at 16 places) would make every store instruction touch 32
+  // rows with 16 bytes each; the tile goes through this wave's private 8 KiB of LDS instead
+  // (16-byte granule XOR row%16: conflict-free both ways) and leaves as whole 256-byte rows,
+  // 16 lanes per row.  lds_wave: this wave's region; out_blk: &out[first row of the wave][head];
+  // rows_valid: how many of the wave's 32 rows exist.
+  __device__ __forceinline__ void store(char *lds_wave, char *out_blk, size_t row_bytes, int rows_valid) {
     const float l_tot = pair_sum(l_run);
     const float inv = (l_tot > 0.0f) ? 1.0f / l_tot : 0.0f;
-    if (!valid) return;
 #pragma unroll
     for (int d = 0; d < 4; ++d)
 #pragma unroll
@@ -297,9 +301,16 @@ template <typename T> struct WaveAttn {
         u32x2_t w;
         w[0] = E::pack2(o[d][4 * i4] * inv, o[d][4 * i4 + 1] * inv);
         w[1] = E::pack2(o[d][4 * i4 + 2] * inv, o[d][4 * i4 + 3] * inv);
-        const int dd = 32 * d + 8 * i4 + 4 * hh;
-        *reinterpret_cast<u32x2_t *>(out_row_head + dd * 2) = w;
+        const int gran = 4 * d + i4;  // 16-byte granule of dims 32d + 8*i4 .. +7; hh picks its half
+        *reinterpret_cast<u32x2_t *>(lds_wave + l32 * kRowBytes + ((gran ^ (l32 & 15)) << 4) + hh * 8) = w;
       }
+    __builtin_amdgcn_wave_barrier();  // wave-private region: LDS ops of one wave complete in order
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const int r = 4 * t + g16;
+      const u32x4_t v = lds_read_b128(lds_wave, r * kRowBytes + ((li ^ (r & 15)) << 4));
+      if (r < rows_valid) *reinterpret_cast<u32x4_t *>(out_blk + (size_t)r * row_bytes + li * 16) = v;
+    }
   }
 };
 
@@ -465,7 +476,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
       if (st == 0 && jb + SUB >= J) break;  // workgroup-uniform: the second stage holds nothing
     }
   }
-  w.store(p.out + (size_t)qrow * q_row_bytes + (size_t)head * kRowBytes, qrow < p.m);
+  // every wave is past the last barrier of the loop: nobody reads the K/V tiles any more
+  w.store(lds + wave * 32 * kRowBytes, p.out + (size_t)qblk0 * q_row_bytes + (size_t)head * kRowBytes, q_row_bytes,
+          p.m - qblk0);
 }
 
 template <typename T, int NW>

@@ -20,7 +20,7 @@
 // O / l rounded once; l sums the ROUNDED probabilities (what P.V used).
 //
 // flash_prefill_kernel<T, NW>: NW waves share the K/V tiles of 32*NW query rows.
-// NW = 8 (one workgroup per CU) once 256-row workgroups alone fill the chip, NW = 4
+// NW = 8 (one workgroup per CU) once there are about 1.5 such workgroups per CU, NW = 4
 // (two workgroups per CU) for smaller problems.  Tiles travel global -> LDS without
 // VGPR staging (global_load_lds_dwordx4), spread over the MFMA stream.  The loop is
 // software pipelined inside a wave: the MFMAs of S(j+1) are issued beside the softmax
@@ -517,6 +517,15 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
   return hipGetLastError();
 }
 
+// 256-row workgroups (one per CU) or 128-row ones (two per CU)?  The 256-row kernel has the
+// cheaper step (K/V tiles shared by twice the rows) but coarser work items: with fewer than
+// about one and a half of them per CU the heavy-first list packs badly (the second round is
+// mostly idle) and the 128-row kernel wins.  Measured at H=28, bf16 (128-row / 256-row, us):
+// S=2560 64/73, S=3072 82/88, S=3584 111/107, S=4096 139/131, S=5120 201/194, S=8192 452/438.
+static bool prefer_256_rows(int m, int H) {
+  return (long long)((m + 255) / 256) * H >= 384;
+}
+
 hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
                                 int n, int offset, int group_size, int kv_head_num, int dt,
                                 hipStream_t stream) {
@@ -532,9 +541,7 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
   p.Hkv = kv_head_num;
   p.H = group_size * kv_head_num;
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
-  // 256-row workgroups once they alone fill the 256 CUs; 128-row ones (two per
-  // CU) for smaller problems.
-  const bool big = (long long)((m + 255) / 256) * p.H >= 256;
+  const bool big = prefer_256_rows(m, p.H);
   if (dt == kDtFloat16)
     return big ? launch_prefill_t<_Float16, 8>(p, stream) : launch_prefill_t<_Float16, 4>(p, stream);
   return big ? launch_prefill_t<__bf16, 8>(p, stream) : launch_prefill_t<__bf16, 4>(p, stream);

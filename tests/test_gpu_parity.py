@@ -110,7 +110,7 @@ def test_flash_attn_gqa_vs_oracle(dt, m, n, offset, H, Hkv):
 def _random_shapes():
     """Seeded shape sweep: every loop-exit case of the prefill kernels (1..11 key tiles per
     workgroup, ragged tails, offsets that put the diagonal anywhere in a tile), both the
-    4-wave and the 8-wave kernel (the latter needs ceil(m/256)*H >= 256)."""
+    4-wave and the 8-wave kernel (the latter needs ceil(m/256)*H >= 384)."""
     rng = np.random.default_rng(20240607)
     shapes = []
     for i in range(36):
@@ -121,7 +121,7 @@ def _random_shapes():
         g = int(rng.choice([1, 2, 5, 7]))
         if big:
             tiles = -(-m // 256)
-            while tiles * Hkv * g < 256:
+            while tiles * Hkv * g < 384:
                 Hkv *= 2
         shapes.append((m, m + offset, offset, Hkv * g, Hkv))
     return shapes
@@ -142,11 +142,11 @@ def test_flash_attn_shape_sweep(idx, shape):
 
 
 @pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
-@pytest.mark.parametrize("H,Hkv", [(4, 2), (64, 8)])
+@pytest.mark.parametrize("H,Hkv", [(4, 2), (96, 8)])
 def test_flash_attn_late_large_scores(dt, H, Hkv):
     """Scores that grow along the key axis: the reference maximum of the online softmax has to
     move many times, late in the key loop (the rescale path of the kernels), for the 4-wave
-    (H=4) and the 8-wave (H=64, m=1024) kernel."""
+    (H=4) and the 8-wave (H=96, m=1024) kernel."""
     ops = _ops()
     m = n = 1024
     q = orc.widen(normal_bits(811, (m, H, 128), dt), dt)

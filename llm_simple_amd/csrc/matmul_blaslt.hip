@@ -35,12 +35,16 @@ struct Plan {
   bool ok = false;
 };
 
-struct Blas {
-  std::mutex mu;
+// One handle, workspace and plan cache per device.
+struct DeviceBlas {
   hipblasLtHandle_t handle = nullptr;
   void *workspace = nullptr;
+  std::map<std::tuple<int, int, int, int, int>, Plan> plans;  // m, n, k, dt, bias
+};
+struct Blas {
+  std::mutex mu;
   static constexpr size_t kWorkspaceBytes = 64u << 20;
-  std::map<std::tuple<int, int, int, int, int, int>, Plan> plans;  // device, m, n, k, dt, bias
+  std::map<int, DeviceBlas> dev;
 };
 
 Blas &blas() {
@@ -50,7 +54,7 @@ Blas &blas() {
 
 hipError_t to_hip(hipblasStatus_t s) { return s == HIPBLAS_STATUS_SUCCESS ? hipSuccess : hipErrorUnknown; }
 
-hipError_t make_plan(Blas &b, Plan &pl, int m, int n, int k, int dt, bool has_bias) {
+hipError_t make_plan(DeviceBlas &b, Plan &pl, int m, int n, int k, int dt, bool has_bias) {
   const hipDataType t = dt == kDtFloat16 ? HIP_R_16F : HIP_R_16BF;
   hipblasStatus_t s = hipblasLtMatmulDescCreate(&pl.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F);
   if (s != HIPBLAS_STATUS_SUCCESS) return to_hip(s);
@@ -86,20 +90,32 @@ hipError_t make_plan(Blas &b, Plan &pl, int m, int n, int k, int dt, bool has_bi
 
 hipError_t launch_matmul_bias(void *out, const void *lhs, const void *weight, const float *bias,
                               int m, int n, int k, int dt, hipStream_t stream) {
-  Blas &b = blas();
-  std::lock_guard<std::mutex> lock(b.mu);
+  Blas &all = blas();
+  std::lock_guard<std::mutex> lock(all.mu);
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
+  DeviceBlas &b = all.dev[dev];
   if (!b.handle) {
     if (hipblasLtCreate(&b.handle) != HIPBLAS_STATUS_SUCCESS) return hipErrorUnknown;
     e = hipMalloc(&b.workspace, Blas::kWorkspaceBytes);
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess) {
+      hipblasLtDestroy(b.handle);
+      b.handle = nullptr;
+      return e;
+    }
   }
-  Plan &pl = b.plans[std::make_tuple(dev, m, n, k, dt, bias ? 1 : 0)];
+  Plan &pl = b.plans[std::make_tuple(m, n, k, dt, bias ? 1 : 0)];
   if (!pl.ok) {
     e = make_plan(b, pl, m, n, k, dt, bias != nullptr);
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess) {  // nothing half-built stays behind
+      if (pl.la) hipblasLtMatrixLayoutDestroy(pl.la);
+      if (pl.lb) hipblasLtMatrixLayoutDestroy(pl.lb);
+      if (pl.lc) hipblasLtMatrixLayoutDestroy(pl.lc);
+      if (pl.desc) hipblasLtMatmulDescDestroy(pl.desc);
+      pl = Plan();
+      return e;
+    }
   }
   if (bias) {
     // the bias pointer is a per-call attribute of the (cached) descriptor; calls are
@@ -114,20 +130,25 @@ hipError_t launch_matmul_bias(void *out, const void *lhs, const void *weight, co
 }
 
 void release_matmul_resources() {
-  Blas &b = blas();
-  std::lock_guard<std::mutex> lock(b.mu);
-  for (auto &kv : b.plans) {
-    Plan &pl = kv.second;
-    if (pl.la) hipblasLtMatrixLayoutDestroy(pl.la);
-    if (pl.lb) hipblasLtMatrixLayoutDestroy(pl.lb);
-    if (pl.lc) hipblasLtMatrixLayoutDestroy(pl.lc);
-    if (pl.desc) hipblasLtMatmulDescDestroy(pl.desc);
+  Blas &all = blas();
+  std::lock_guard<std::mutex> lock(all.mu);
+  int cur = 0;
+  const bool have_cur = hipGetDevice(&cur) == hipSuccess;
+  for (auto &dv : all.dev) {
+    DeviceBlas &b = dv.second;
+    (void)hipSetDevice(dv.first);
+    for (auto &kv : b.plans) {
+      Plan &pl = kv.second;
+      if (pl.la) hipblasLtMatrixLayoutDestroy(pl.la);
+      if (pl.lb) hipblasLtMatrixLayoutDestroy(pl.lb);
+      if (pl.lc) hipblasLtMatrixLayoutDestroy(pl.lc);
+      if (pl.desc) hipblasLtMatmulDescDestroy(pl.desc);
+    }
+    if (b.workspace) (void)hipFree(b.workspace);
+    if (b.handle) hipblasLtDestroy(b.handle);
   }
-  b.plans.clear();
-  if (b.workspace) (void)hipFree(b.workspace);
-  b.workspace = nullptr;
-  if (b.handle) hipblasLtDestroy(b.handle);
-  b.handle = nullptr;
+  all.dev.clear();
+  if (have_cur) (void)hipSetDevice(cur);
 }
 
 // out = round_T(float(lhs) + float(rhs)), 8 elements per thread (HBM-bound: 6 bytes per element).

@@ -29,6 +29,8 @@
 // Every LDS fragment address is a loop-invariant register plus an immediate, and a
 // tile load is a scalar base plus a loop-invariant lane offset: the loop spends its
 // vector ALU instructions on the softmax only.
+#include <atomic>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -505,13 +507,17 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
   }
   const size_t lds_bytes = (NW == 8 ? 2 : 1) * 4 * kTileBytes;
   void (*kern)(PrefillParams) = flash_prefill_kernel<T, NW>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes);
+  // the opt-in for more than 64 KiB of dynamic LDS is per device: once per device and kernel
+  static std::atomic<uint64_t> attr_done{0};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (!(attr_done.load(std::memory_order_acquire) & bit)) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
-    attr_set = true;
+    attr_done.fetch_or(bit, std::memory_order_release);
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds_bytes, stream, p);
   return hipGetLastError();

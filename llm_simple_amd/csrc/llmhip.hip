@@ -59,6 +59,8 @@ int attn_common(void *out, const void *q, const void *k, const void *v, int m, i
     return LLMHIP_ERR_INVALID_ARG;
   if (!dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
   if (head_dim != 128) return LLMHIP_ERR_UNSUPPORTED;
+  // grid dimensions and the 32-bit row offsets of the tile loader
+  if (kv_head_num > 65535 || (long long)group_size * kv_head_num > 65535) return LLMHIP_ERR_UNSUPPORTED;
   if ((long long)m * group_size <= kMaxDecodeCols) {
     // few query rows: stream the cache once with the split-KV kernel
     const int n_vis = (n < m + offset) ? n : m + offset;  // keys any row can see

@@ -15,7 +15,9 @@ reference's CPU layer attention, src/llama2_layer_cpu.cpp:175-296) on the host
 cores as a reported baseline.
 
 Launch durations are measured with HIP events recorded on the stream the
-kernels run on (the default stream), around back-to-back launches.
+kernels run on (the default stream), around back-to-back launches.  The default
+run is long enough for the clocks to settle (the first ~50 ms of a burst run
+about 8 % slower than the sustained rate).
 """
 import argparse
 import json
@@ -235,8 +237,8 @@ def cpu_baseline(S, H=28, Hkv=4):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--seq", type=int, default=4096, help="prefill sequence length of the timed step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="comma list of legs: prefill,decode,rope,block (default all)")
@@ -272,7 +274,7 @@ def main():
         for S in (1024, 8192):
             if S == args.seq:
                 continue
-            r, _ = bench_prefill(ops, torch, timer, S, max(10, args.steps // 4), 5)
+            r, _ = bench_prefill(ops, torch, timer, S, max(10, args.steps // 4), max(5, args.warmup // 4))
             log(f"prefill S={S}: {r['ms_event'] * 1e3:.1f} us  {r['tflops']:.1f} TFLOP/s")
             others.append({"S": S, "us": r["ms_event"] * 1e3, "tflops": r["tflops"],
                            "frac": r["tflops"] / PEAK_BF16_TFLOPS})

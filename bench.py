@@ -37,7 +37,7 @@ DT_BF16 = 5
 # scaled by 2.000 and WRITE_SIZE by 1.000, the factors a plain 1 GiB copy gives); the commands and raw
 # figures are in profiles/.  Only the shapes that were profiled have an entry.
 MEASURED_TRAFFIC_BYTES = {
-    ("prefill", 4096): (47117 + 28672) * 1024,             # algorithmic 65536 KiB
+    ("prefill", 4096): (47128 + 28672) * 1024,             # algorithmic 65536 KiB
     ("decode", 16, 32768): (2097572 + 656) * 1024,         # algorithmic 2097152 KiB
     ("decode", 1, 32768): (131250 + 656) * 1024,           # algorithmic 131072 KiB
     ("rope", 4096): (40530 + 36864) * 1024,                # algorithmic 75776 KiB

@@ -75,3 +75,20 @@ def test_matmul_rejects_bad_arguments():
         ops.hip_matmul_layer(out, x, w, 4, 16, 32, 7)             # unknown dtype
     with pytest.raises(ops.LlmHipError):
         ops.hip_matmul_layer(out, x, w, 0, 16, 32, DT_BFLOAT16)   # m < 1
+
+
+def test_release_then_reuse():
+    """llmhip_release_internal_workspace() drops the hipBLASLt handle, plans and workspace (and the
+    decode scratch); the next call builds them again."""
+    ops = _ops()
+    dt, m, n, k = DT_BFLOAT16, 8, 64, 128
+    x = normal_bits(21, (m, k), dt)
+    w = orc.round_to(orc.widen(normal_bits(22, (n, k), dt), dt) / np.sqrt(k), dt)
+    ref = orc.widen(orc.matmul_bias(x, w, None, dt), dt)
+    for _ in range(2):
+        d_out = dev_empty((m, n))
+        ops.hip_matmul_layer(d_out, to_dev(x), to_dev(w), m, n, k, dt)
+        got = orc.widen(to_host(d_out), dt)
+        assert (np.abs(got - ref) <= np.maximum(1.01 * ulp(ref, dt), 1e-3)).all()
+        assert ops.lib.llmhip_device_sync() == 0
+        assert ops.lib.llmhip_release_internal_workspace() == 0

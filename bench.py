@@ -5,10 +5,10 @@
 
 A "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM: the causal flash-attention prefill launch at
-BASELINE.json's Qwen2.5-7B shape (bf16, H=28, Hkv=4, head_dim 128, S=4096).
+the headline benchmark shape, Qwen2.5-7B (bf16, H=28, Hkv=4, head_dim 128, S=4096).
 `value` is its algorithmic throughput, 4*H*hd*S(S+1)/2 FLOP per launch over the
 measured time per launch.  The same run also measures the two other kernels of
-the path at their BASELINE shapes -- split-KV decode at the Qwen2.5-32B shape
+the path at their benchmark shapes -- split-KV decode at the Qwen2.5-32B shape
 (H=40, Hkv=8, KV length 32768, batch 1 and 16; algorithmic bytes = K and V read
 once) and the fused RoPE + KV append -- and times the CPU oracle (a port of the
 reference's CPU layer attention, src/llama2_layer_cpu.cpp:175-296) on the host
@@ -251,7 +251,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU; --gpus must be 1 "
-            "(the path shards by kv head without any exchange, see DESIGN.md)")
+            "(the path shards by kv head without any exchange between GPUs)")
         sys.exit(2)
 
     import torch
@@ -345,8 +345,8 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"Qwen2.5-7B causal prefill attention, bf16, batch 1, H=28, Hkv=4, "
-                               f"head_dim=128, S={args.seq} (BASELINE configs[3]); decode leg: "
-                               f"Qwen2.5-32B H=40 Hkv=8 n=32768 (configs[4])"},
+                               f"head_dim=128, S={args.seq} (benchmark configuration 4); decode leg: "
+                               f"Qwen2.5-32B H=40 Hkv=8 n=32768 (benchmark configuration 5)"},
         "roofline": {"bound": "mfma", "achieved": pre["tflops"], "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": pre["tflops"] / PEAK_BF16_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(("prefill", args.seq)),

@@ -48,7 +48,7 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None, layer_style=Tr
     """Compare HIP output bits with both oracles.
 
     Against the fp32 oracle (the reference's test golden): max-abs <= TOL, the
-    bar BASELINE sets.  Against the layer-style oracle, whose output is itself
+    bar of the benchmark definition.  Against the layer-style oracle, whose output is itself
     rounded to the storage type: fp16 (the arithmetic the reference's CPU layer
     really has) within TOL or two representable steps for all but at most one element
     per million; bf16 (no reference code,

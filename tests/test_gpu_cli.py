@@ -19,7 +19,7 @@ def _run(exe, *flags):
 
 
 @pytest.mark.parametrize("flags", [
-    ("--m", 256, "--n", 256, "--offset", 0, "--head_num", 32, "--head_dim", 128),                 # BASELINE config 1
+    ("--m", 256, "--n", 256, "--offset", 0, "--head_num", 32, "--head_dim", 128),                 # benchmark configuration 1
     ("--m", 1, "--n", 512, "--offset", 511, "--head_num", 32),                                    # config 2
     ("--m", 256, "--n", 256, "--head_num", 12, "--kv_head_num", 2, "--dtype", "bf16"),            # config 3 prefill
     ("--m", 1024, "--n", 1024, "--head_num", 28, "--kv_head_num", 4, "--dtype", "bf16"),          # config 4, S=1024

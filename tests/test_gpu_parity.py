@@ -161,7 +161,7 @@ def test_flash_attn_late_large_scores(dt, H, Hkv):
 
 
 def test_llama2_prefill_config_fp16():
-    """BASELINE config 1: Llama2-7B prefill, fp16, H = Hkv = 32, m = n = 256, through the
+    """Benchmark configuration 1: Llama2-7B prefill, fp16, H = Hkv = 32, m = n = 256, through the
     MHA entry point and the reference's own tolerance rule
     (tests/npu_op_test_util.cpp:33-48: abs 1e-3 AND rel 1e-3)."""
     ops = _ops()
@@ -179,7 +179,7 @@ def test_llama2_prefill_config_fp16():
 
 
 def test_llama2_decode_config_fp16():
-    """BASELINE config 2: one query token over a 512-row fp16 cache, H = Hkv = 32."""
+    """Benchmark configuration 2: one query token over a 512-row fp16 cache, H = Hkv = 32."""
     ops = _ops()
     dt, H, n = DT_FLOAT16, 32, 512
     q = normal_bits(2001, (1, H, 128), dt)
@@ -216,7 +216,7 @@ def test_flash_decode_splits(dt, splits, batch, n, stride, H, Hkv):
 
 @pytest.mark.parametrize("S,rows_per_probe", [(2400, 24), (4096, 16)])
 def test_qwen7b_prefill_full_size_sampled(S, rows_per_probe):
-    """BASELINE config 4 shape (H=28, Hkv=4, bf16) at sizes the CPU oracle cannot
+    """Benchmark configuration 4 shape (H=28, Hkv=4, bf16) at sizes the CPU oracle cannot
     finish whole: every sampled output row is checked against the oracle run as a
     one-row decode over the same keys (row r of a causal prefill == decode with
     n = r + 1)."""
@@ -240,7 +240,7 @@ def test_qwen7b_prefill_full_size_sampled(S, rows_per_probe):
 
 
 def test_qwen15b_config_prefill_then_256_decode_steps():
-    """BASELINE config 3: Qwen2.5-1.5B, H=12, Hkv=2, bf16, theta 1e6 (table rounded to bf16,
+    """Benchmark configuration 3: Qwen2.5-1.5B, H=12, Hkv=2, bf16, theta 1e6 (table rounded to bf16,
     src/model_base.cpp:59-66), neox RoPE, QKV bias ~ N(0, 0.02) in fp32 added before the single
     rounding to bf16 (the projection epilogue, tests/gemm_test.cpp:138-149); prefill of 256 tokens,
     then 256 decode steps with the KV cache growing in place 256 -> 512.  Every step runs the fused
@@ -283,7 +283,7 @@ def test_qwen15b_config_prefill_then_256_decode_steps():
 
 @pytest.mark.parametrize("batch,n", [(1, 32768), (16, 4096)])
 def test_qwen32b_decode_full_size(batch, n):
-    """BASELINE config 5 shape (H=40, Hkv=8, bf16) at full KV length: the CPU oracle streams the
+    """Benchmark configuration 5 shape (H=40, Hkv=8, bf16) at full KV length: the CPU oracle streams the
     same caches (decode is cheap on the CPU); plus two size-independent properties: a joint
     permutation of the (K, V) rows leaves the output unchanged up to rounding, and the result
     does not depend on the split count."""

@@ -345,8 +345,8 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"Qwen2.5-7B causal prefill attention, bf16, batch 1, H=28, Hkv=4, "
-                               f"head_dim=128, S={args.seq} (benchmark configuration 4); decode leg: "
-                               f"Qwen2.5-32B H=40 Hkv=8 n=32768 (benchmark configuration 5)"},
+                               f"head_dim=128, S={args.seq} (BASELINE.json configs[3]); decode leg: "
+                               f"Qwen2.5-32B H=40 Hkv=8 n=32768 (BASELINE.json configs[4])"},
         "roofline": {"bound": "mfma", "achieved": pre["tflops"], "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": pre["tflops"] / PEAK_BF16_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(("prefill", args.seq)),

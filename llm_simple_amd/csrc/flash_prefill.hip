@@ -17,7 +17,7 @@
 // read with ds_read_b128, V^T fragments with ds_read_b64_tr_b16.  exp2 with the
 // scale folded into one FMA; the reference maximum is kept in raw score units and
 // moves lazily, so O is rarely rescaled.  Accumulation is fp32; out =
-// O / l rounded once; l sums the probabilities in fp32 before they are rounded for P.V.
+// O / l rounded once; l sums the ROUNDED probabilities (what P.V used).
 //
 // flash_prefill_kernel<T, NW>: NW waves share the K/V tiles of 32*NW query rows.
 // NW = 8 (one workgroup per CU) once there are about 1.5 such workgroups per CU, NW = 4
@@ -106,6 +106,19 @@ __device__ __forceinline__ float pair_sum(float x) {
   float lo, hi;
   pair_swap(x, lo, hi);
   return lo + hi;
+}
+
+// acc + lo + hi of a packed pair of storage-type values.
+template <typename T> __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc);
+template <> __device__ __forceinline__ float dot2_ones<__bf16>(uint32_t packed, float acc) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 b2;
+  const b2 one = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, packed), one, acc, false);
+}
+template <> __device__ __forceinline__ float dot2_ones<_Float16>(uint32_t packed, float acc) {
+  typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+  const h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), one, acc, false);
 }
 
 // LDS visibility + workgroup barrier that does not drain outstanding global loads.
@@ -222,7 +235,7 @@ template <typename T> struct WaveAttn {
   }
 
   // P = exp2(s*c + neg_ms) rounded to T and packed as the B operand; returns this lane's sum
-  // of the (unrounded) values.
+  // of the rounded values.
   __device__ __forceinline__ float probabilities(const f32x16_t (&s)[2], float c, float neg_ms) {
     float ps0 = 0.0f, ps1 = 0.0f;
 #pragma unroll
@@ -235,12 +248,16 @@ template <typename T> struct WaveAttn {
           const float e0 = fast_exp2(__builtin_fmaf(s[kb][8 * ks2 + 2 * e2], c, neg_ms));
           const float e1 = fast_exp2(__builtin_fmaf(s[kb][8 * ks2 + 2 * e2 + 1], c, neg_ms));
           w[e2] = E::pack2(e0, e1);
-          // plain fp32 adds: v_dot2_f32_bf16 / v_dot2_f32_f16 on the packed pair would sum the
-          // rounded values in one instruction, but dot instructions queue behind the MFMAs of
-          // every wave on the SIMD (a softmax pass beside an MFMA-issuing wave: 1690 cycles
-          // with them, 1070 without)
-          ps0 += e0;
-          ps1 += e1;
+          // l sums the ROUNDED probabilities, the values P.V really used: for rows that see few
+          // keys the rounding errors of numerator and denominator then cancel.  (In a design that
+          // separates MFMA and softmax phases these dot instructions are costly -- they queue
+          // behind the MFMAs of every wave on the SIMD: a softmax pass beside an MFMA-issuing wave
+          // takes 1690 cycles with them, 1070 with plain adds -- in this interleaved loop the
+          // two versions time the same.)
+          if (e2 & 1)
+            ps1 = dot2_ones<T>(w[e2], ps1);
+          else
+            ps0 = dot2_ones<T>(w[e2], ps0);
         }
         pf[kb][ks2] = w;
       }

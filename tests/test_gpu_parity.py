@@ -311,3 +311,19 @@ def test_qwen32b_decode_full_size(batch, n):
     assert np.abs(orc.widen(out, dt) - orc.widen(out_p, dt)).max() <= 2 * 2.0 ** -8
     out_s = run(k, v, 7)
     assert np.abs(orc.widen(out, dt) - orc.widen(out_s, dt)).max() <= 2 * 2.0 ** -8
+
+
+def test_long_context_131072():
+    """A 131072-token cache (the longest context Qwen2.5 advertises) at the 32B head counts: one decode
+    step and a 40-token chunk appended at the end (the prefill kernel walking 2048 key tiles), against
+    the oracle.  Guards the 32/64-bit address arithmetic of both kernels."""
+    ops = _ops()
+    dt, H, Hkv, n = DT_BFLOAT16, 40, 8, 131072
+    k = normal_bits(1301, (n, Hkv, 128), dt)
+    v = normal_bits(1302, (n, Hkv, 128), dt)
+    dk, dv = to_dev(k), to_dev(v)
+    for m in (1, 40):
+        q = normal_bits(1300 + m, (m, H, 128), dt)
+        d_out = dev_empty(q.shape)
+        ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), dk, dv, m, n, n - m, H // Hkv, Hkv, 128, dt)
+        check_attention(to_host(d_out), q, k, v, n, n - m, dt)

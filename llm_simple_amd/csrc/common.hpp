@@ -85,6 +85,19 @@ __device__ __forceinline__ float xor_lane(float v, int mask) { return __shfl_xor
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// acc + lo + hi of a packed pair of storage-type values.
+template <typename T> __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc);
+template <> __device__ __forceinline__ float dot2_ones<__bf16>(uint32_t packed, float acc) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 b2;
+  const b2 one = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, packed), one, acc, false);
+}
+template <> __device__ __forceinline__ float dot2_ones<_Float16>(uint32_t packed, float acc) {
+  typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+  const h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), one, acc, false);
+}
+
 // LDS tile of 16-bit head rows, 256 bytes per row, 16 granules of 16 bytes.
 // K tiles are read with ds_read_b128 by 16 consecutive rows at one logical
 // granule: XOR with the row spreads them over all 16 bank groups.

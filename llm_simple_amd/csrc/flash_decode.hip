@@ -161,22 +161,23 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
       const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
       const float alpha = fast_exp2(m_run - m_use);
       m_run = m_new;
-      float psum = 0.0f;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float e = fast_exp2(s[blk][i] - m_use);
-          s[blk][i] = e;
-          psum += e;
-        }
-      l_run = l_run * alpha + psum;
+        for (int i = 0; i < 4; ++i) s[blk][i] = fast_exp2(s[blk][i] - m_use);
       // P^T as B operand: slot e<4 -> block 0 key 4cg+e, e>=4 -> block 1 key 4cg+e-4
       u32x4_t pf;
       pf[0] = E::pack2(s[0][0], s[0][1]);
       pf[1] = E::pack2(s[0][2], s[0][3]);
       pf[2] = E::pack2(s[1][0], s[1][1]);
       pf[3] = E::pack2(s[1][2], s[1][3]);
+      // the row sum takes the ROUNDED probabilities, the values P.V uses: numerator and
+      // denominator then carry the same rounding (as in the prefill kernel)
+      float psum = dot2_ones<T>(pf[0], 0.0f);
+      psum = dot2_ones<T>(pf[1], psum);
+      psum = dot2_ones<T>(pf[2], psum);
+      psum = dot2_ones<T>(pf[3], psum);
+      l_run = l_run * alpha + psum;
       // ---- O^T += V^T P^T ----
       const int vr = 4 * cg + (col >> 2);
       const int sub = (col & 1) * 8;

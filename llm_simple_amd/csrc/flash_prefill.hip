@@ -108,19 +108,6 @@ __device__ __forceinline__ float pair_sum(float x) {
   return lo + hi;
 }
 
-// acc + lo + hi of a packed pair of storage-type values.
-template <typename T> __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc);
-template <> __device__ __forceinline__ float dot2_ones<__bf16>(uint32_t packed, float acc) {
-  typedef __attribute__((ext_vector_type(2))) __bf16 b2;
-  const b2 one = {(__bf16)1.0f, (__bf16)1.0f};
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, packed), one, acc, false);
-}
-template <> __device__ __forceinline__ float dot2_ones<_Float16>(uint32_t packed, float acc) {
-  typedef __attribute__((ext_vector_type(2))) _Float16 h2;
-  const h2 one = {(_Float16)1.0f, (_Float16)1.0f};
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), one, acc, false);
-}
-
 // LDS visibility + workgroup barrier that does not drain outstanding global loads.
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");

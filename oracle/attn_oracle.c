@@ -24,6 +24,14 @@
  *   orc_attention_f32 / orc_attention_layer
  *                          pinned for MHA: textbook SDPA (torch, fp64), fp64
  *                          brute force, softmax invariants.
+ *                          The three rounding points of orc_attention_layer
+ *                          (scores after the scale, probabilities after the
+ *                          division, output) are pinned by hand-derived bit
+ *                          patterns on 2..11-key cases with exact dot products
+ *                          (tests/test_oracle_layer_rounding.py): a chain that
+ *                          drops one, moves the probability rounding before
+ *                          the division or rounds to the other 16-bit type
+ *                          misses at least one of them.
  *                          GQA head mapping (kv = h / group_size) and the bf16
  *                          variant have no reference CPU code and no reference
  *                          test: PARITY UNPINNED against the reference at that

@@ -51,10 +51,10 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None, layer_style=Tr
     bar of the benchmark definition.  Against the layer-style oracle, whose output is itself
     rounded to the storage type: fp16 (the arithmetic the reference's CPU layer
     really has) within TOL or two representable steps for all but at most one element
-    per million; bf16 (no reference code,
-    the same chain with bf16 casts, which by itself sits up to ~1.2e-2 from the
-    fp32 oracle on rows that see few keys, tests/test_oracle_attention.py) within
-    TOL plus that oracle's own distance from the fp32 one.  layer_style=False skips the second
+    per million; bf16 (no reference code, the same chain with bf16 casts, which by itself
+    sits up to ~1.2e-2 from the fp32 oracle on rows that see few keys,
+    tests/test_oracle_attention.py) within TOL or two steps for all but 200 elements per
+    million and within TOL or three steps for all but 2 per million.  layer_style=False skips the second
     comparison: for scores of magnitude ~30 the layer-style chain's rounding of the scores to
     fp16 alone (steps of 2^-6) moves the probabilities by more than TOL."""
     got = orc.widen(out_bits, dt)
@@ -71,12 +71,18 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None, layer_style=Tr
         return e32, None
     assert e32 <= TOL[dt], f"max-abs vs fp32 oracle {e32} > {TOL[dt]}"
     d16 = np.abs(got - ref16)
-    # nothing can be further from the layer-style oracle than the bound above plus that oracle's own
-    # distance from the fp32 one ...
-    assert (d16 <= TOL[dt] + np.abs(ref16 - ref32) + 1e-7).all(), f"worst {d16.max()}"
+    u = ulp(ref16, dt)
+    near = lambda steps: np.count_nonzero(~((d16 <= TOL[dt]) | (d16 <= (steps + 1e-4) * u)))
     if dt == DT_FLOAT16:
-        # ... and for fp16, the arithmetic the reference's CPU layer really has, all but a few
-        # elements per million sit within TOL or two representable steps of it
-        off = np.count_nonzero(~((d16 <= TOL[dt]) | (d16 <= 2.0001 * ulp(ref16, dt))))
+        # fp16 is the arithmetic the reference's CPU layer really has: all but one element per million sit
+        # within TOL or two representable steps of it
+        off = near(2)
         assert off <= max(1, got.size // 10 ** 6), f"{off} elements off the layer-style oracle, worst {d16.max()}"
+    else:
+        # bf16: the layer-style chain rounds scores and probabilities to 8 bits, so single elements of rows
+        # that see few keys land a step or two further away (measured on the kernels over 27 shapes: at most
+        # 76 per million beyond TOL-or-2-steps, at most 0.3 per million beyond TOL-or-3-steps)
+        off2, off3 = near(2), near(3)
+        assert off2 <= max(2, got.size * 200 // 10 ** 6), f"{off2} of {got.size} elements beyond 2 steps, worst {d16.max()}"
+        assert off3 <= max(1, got.size * 2 // 10 ** 6), f"{off3} of {got.size} elements beyond 3 steps, worst {d16.max()}"
     return e32, float(d16.max())

@@ -90,6 +90,10 @@ ATTN_CASES = [
     (300, 300, 0, 28, 4),
     (77, 590, 513, 28, 4),
     (513, 513, 0, 5, 5),
+    # n < m + offset: the cache length, not the causal bound, cuts the last rows
+    (40, 50, 30, 4, 2),
+    (300, 320, 100, 8, 2),
+    (9, 10, 5, 2, 1),
 ]
 
 
@@ -178,6 +182,54 @@ def test_llama2_prefill_config_fp16():
         assert bad == 0
 
 
+def test_llama2_prefill_then_decode_chain_fp16():
+    """Benchmark configurations 1 and 2 through the whole path at full shape: Llama2-7B, fp16, H = Hkv = 32,
+    theta 10000, interleaved RoPE (src/llama2_main.cpp:123-126).  Prefill: 256 tokens rotated, appended
+    at rows 0..255, attended.  Decode: a cache of 511 rows, the new token rotated at position 511 and
+    appended at row 511, attention m=1, n=512, offset=511.  Rotated Q and both caches bit-exact, the
+    attention output against both oracles and the reference's all_close rule."""
+    ops = _ops()
+    dt, H, max_seq = DT_FLOAT16, 32, 512
+    table = orc.init_freq_cis(128, max_seq, 10000.0, dt)
+    d_table = f32_dev(table)
+    # --- config 1
+    m = 256
+    q, k, v = (normal_bits(1001 + i, (m, H, 128), dt) for i in range(3))
+    kc = np.full((max_seq, H, 128), 0x7FFF, dtype=np.uint16)  # NaN patterns: rows >= n must not be read
+    vc = kc.copy()
+    d_q, d_kc, d_vc, d_o = dev_empty(q.shape), to_dev(kc), to_dev(vc), dev_empty(q.shape)
+    ops.hip_rope_kv_append_layer(d_q, d_kc, d_vc, d_table, to_dev(q), to_dev(k), to_dev(v), 0, m, H, H, 128,
+                                 False, dt)
+    ops.hip_flash_attn_layer(d_o, d_q, d_kc, d_vc, m, m, 0, H, 128, dt)
+    q_r = orc.rope(q, table, 0, False, dt)
+    orc.kv_append(kc, orc.rope(k, table, 0, False, dt), 0)
+    orc.kv_append(vc, v, 0)
+    assert np.array_equal(to_host(d_q), q_r)
+    assert np.array_equal(to_host(d_kc), kc) and np.array_equal(to_host(d_vc), vc)
+    out = to_host(d_o)
+    check_attention(out, q_r, kc, vc, m, 0, dt)
+    bad, _ = orc.all_close(orc.widen(out, dt), orc.attention_f32(q_r, kc, vc, m, 0, dt))
+    assert bad == 0
+    # --- config 2: rows 256..510 are "generated" tokens already in the cache
+    kc[m:511] = normal_bits(1002, (511 - m, H, 128), dt)
+    vc[m:511] = normal_bits(1012, (511 - m, H, 128), dt)
+    d_kc, d_vc = to_dev(kc), to_dev(vc)
+    q1, k1, v1 = (normal_bits(1020 + i, (1, H, 128), dt) for i in range(3))
+    d_q1, d_o1 = dev_empty(q1.shape), dev_empty(q1.shape)
+    ops.hip_rope_kv_append_layer(d_q1, d_kc, d_vc, d_table, to_dev(q1), to_dev(k1), to_dev(v1), 511, 1, H, H,
+                                 128, False, dt)
+    ops.hip_flash_attn_layer(d_o1, d_q1, d_kc, d_vc, 1, 512, 511, H, 128, dt)
+    q1_r = orc.rope(q1, table, 511, False, dt)
+    orc.kv_append(kc, orc.rope(k1, table, 511, False, dt), 511)
+    orc.kv_append(vc, v1, 511)
+    assert np.array_equal(to_host(d_q1), q1_r)
+    assert np.array_equal(to_host(d_kc), kc) and np.array_equal(to_host(d_vc), vc)
+    out1 = to_host(d_o1)
+    check_attention(out1, q1_r, kc, vc, 512, 511, dt)
+    bad, _ = orc.all_close(orc.widen(out1, dt), orc.attention_f32(q1_r, kc, vc, 512, 511, dt))
+    assert bad == 0
+
+
 def test_llama2_decode_config_fp16():
     """Benchmark configuration 2: one query token over a 512-row fp16 cache, H = Hkv = 32."""
     ops = _ops()
@@ -214,7 +266,7 @@ def test_flash_decode_splits(dt, splits, batch, n, stride, H, Hkv):
     check_attention(to_host(d_out), q, k, v, n, n - 1, dt, batch=True)
 
 
-@pytest.mark.parametrize("S,rows_per_probe", [(2400, 24), (4096, 16)])
+@pytest.mark.parametrize("S,rows_per_probe", [(1024, 24), (2400, 24), (4096, 16), (8192, 12)])
 def test_qwen7b_prefill_full_size_sampled(S, rows_per_probe):
     """Benchmark configuration 4 shape (H=28, Hkv=4, bf16) at sizes the CPU oracle cannot
     finish whole: every sampled output row is checked against the oracle run as a
@@ -239,9 +291,11 @@ def test_qwen7b_prefill_full_size_sampled(S, rows_per_probe):
     assert np.isfinite(orc.widen(out, dt)).all()
 
 
-def test_qwen15b_config_prefill_then_256_decode_steps():
+@pytest.mark.parametrize("is_neox", [True, False])
+def test_qwen15b_config_prefill_then_256_decode_steps(is_neox):
     """Benchmark configuration 3: Qwen2.5-1.5B, H=12, Hkv=2, bf16, theta 1e6 (table rounded to bf16,
-    src/model_base.cpp:59-66), neox RoPE, QKV bias ~ N(0, 0.02) in fp32 added before the single
+    src/model_base.cpp:59-66), neox RoPE as the Qwen recipes run it (scripts/benchmark_qwen2.5.sh:12) and
+    also interleaved, QKV bias ~ N(0, 0.02) in fp32 added before the single
     rounding to bf16 (the projection epilogue, tests/gemm_test.cpp:138-149); prefill of 256 tokens,
     then 256 decode steps with the KV cache growing in place 256 -> 512.  Every step runs the fused
     rope + append and the attention entry point; every step is checked against the oracle."""
@@ -267,10 +321,10 @@ def test_qwen15b_config_prefill_then_256_decode_steps():
         q, k, v = projected(m, H, "q"), projected(m, Hkv, "k"), projected(m, Hkv, "v")
         d_q, d_o = dev_empty((m, H, 128)), dev_empty((m, H, 128))
         ops.hip_rope_kv_append_layer(d_q, d_kc, d_vc, d_table, to_dev(q), to_dev(k), to_dev(v), prev, m, H,
-                                     Hkv, 128, True, dt)
+                                     Hkv, 128, is_neox, dt)
         ops.hip_flash_attn_gqa_layer(d_o, d_q, d_kc, d_vc, m, cur, prev, H // Hkv, Hkv, 128, dt)
-        q_r = orc.rope(q, table, prev, True, dt)
-        orc.kv_append(kc, orc.rope(k, table, prev, True, dt), prev)
+        q_r = orc.rope(q, table, prev, is_neox, dt)
+        orc.kv_append(kc, orc.rope(k, table, prev, is_neox, dt), prev)
         orc.kv_append(vc, v, prev)
         ref = orc.attention_f32(q_r, kc, vc, cur, prev, dt)
         err = float(np.abs(orc.widen(to_host(d_o), dt) - ref).max())
@@ -281,36 +335,48 @@ def test_qwen15b_config_prefill_then_256_decode_steps():
     assert np.array_equal(to_host(d_kc), kc) and np.array_equal(to_host(d_vc), vc)
 
 
-@pytest.mark.parametrize("batch,n", [(1, 32768), (16, 4096)])
+@pytest.mark.parametrize("batch,n", [(1, 4096), (1, 16384), (1, 32768), (16, 4096), (16, 16384), (16, 32768)])
 def test_qwen32b_decode_full_size(batch, n):
-    """Benchmark configuration 5 shape (H=40, Hkv=8, bf16) at full KV length: the CPU oracle streams the
-    same caches (decode is cheap on the CPU); plus two size-independent properties: a joint
-    permutation of the (K, V) rows leaves the output unchanged up to rounding, and the result
-    does not depend on the split count."""
+    """Benchmark configuration 5 (H=40, Hkv=8, bf16), every KV length and batch size of the benchmark, at
+    full size.  The CPU oracle streams the same caches (all sequences up to 256 MiB of K+V per launch,
+    sequences 0, 7 and 15 of the larger ones); plus two size-independent properties: the result does
+    not depend on the split count, and (up to 256 MiB) a joint permutation of the (K, V) rows leaves
+    the output unchanged up to rounding."""
     import torch
     ops = _ops()
     dt, H, Hkv = DT_BFLOAT16, 40, 8
-    q = normal_bits(1005, (batch, 1, H, 128), dt)
-    k = normal_bits(1006, (batch, n, Hkv, 128), dt)
-    v = normal_bits(1007, (batch, n, Hkv, 128), dt)
     g = H // Hkv
+    q = normal_bits(1005, (batch, 1, H, 128), dt)
+    # the caches are generated one sequence at a time (a 2 GiB launch would need 8 GiB of fp32 normals)
+    k = np.empty((batch, n, Hkv, 128), dtype=np.uint16)
+    v = np.empty_like(k)
+    for b in range(batch):
+        k[b] = normal_bits(1006 + 2 * b, (n, Hkv, 128), dt)
+        v[b] = normal_bits(1007 + 2 * b, (n, Hkv, 128), dt)
+    dk, dv = to_dev(k), to_dev(v)
+    dq = to_dev(q)
 
-    def run(kk, vv, splits):
+    def run(d_k, d_v, splits):
         ns = splits if splits > 0 else ops.flash_decode_default_splits(batch, n, Hkv)
         wsb = ops.flash_decode_workspace_bytes(batch, g, Hkv, 128, ns)
         ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
         d_out = dev_empty((batch, 1, H, 128))
-        ops.hip_flash_decode_gqa_layer(d_out, to_dev(q), to_dev(kk), to_dev(vv), ws, wsb, batch, n, n, g, Hkv,
-                                       128, splits, dt)
+        ops.hip_flash_decode_gqa_layer(d_out, dq, d_k, d_v, ws, wsb, batch, n, n, g, Hkv, 128, splits, dt)
         return to_host(d_out)
 
-    out = run(k, v, 0)
-    check_attention(out, q, k, v, n, n - 1, dt, batch=True)
-    perm = np.random.default_rng(9).permutation(n)
-    out_p = run(np.ascontiguousarray(k[:, perm]), np.ascontiguousarray(v[:, perm]), 0)
-    assert np.abs(orc.widen(out, dt) - orc.widen(out_p, dt)).max() <= 2 * 2.0 ** -8
-    out_s = run(k, v, 7)
+    out = run(dk, dv, 0)
+    small = 2 * k.nbytes <= 256 << 20
+    if small:
+        check_attention(out, q, k, v, n, n - 1, dt, batch=True)
+    else:
+        for b in sorted({0, 7 % batch, batch - 1}):
+            check_attention(out[b], q[b], k[b], v[b], n, n - 1, dt)
+    out_s = run(dk, dv, 7)
     assert np.abs(orc.widen(out, dt) - orc.widen(out_s, dt)).max() <= 2 * 2.0 ** -8
+    if small:
+        perm = np.random.default_rng(9).permutation(n)
+        out_p = run(to_dev(np.ascontiguousarray(k[:, perm])), to_dev(np.ascontiguousarray(v[:, perm])), 0)
+        assert np.abs(orc.widen(out, dt) - orc.widen(out_p, dt)).max() <= 2 * 2.0 ** -8
 
 
 def test_long_context_131072():

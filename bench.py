@@ -15,9 +15,12 @@ reference's CPU layer attention, src/llama2_layer_cpu.cpp:175-296) on the host
 cores as a reported baseline.
 
 Launch durations are measured with HIP events recorded on the stream the
-kernels run on (the default stream), around back-to-back launches.  The default
-run is long enough for the clocks to settle (the first ~50 ms of a burst run
-about 8 % slower than the sustained rate).
+kernels run on (the default stream), around back-to-back launches.  Whatever
+--steps/--warmup say, every leg first launches for at least 100 ms so that the
+clocks settle (the first ~50 ms of a burst run about 8 % slower than the
+sustained rate; reported as settle_ms), then takes the median of 5 batches of
+max(steps, 100) launches.  After the timed region the outputs of the timed
+launches are compared with the CPU oracle on sampled rows (max_abs_err).
 """
 import argparse
 import json
@@ -36,6 +39,7 @@ DT_BF16 = 5
 # HBM bytes per launch read off rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, FETCH_SIZE
 # scaled by 2.000 and WRITE_SIZE by 1.000, the factors a plain 1 GiB copy gives); the commands and raw
 # figures are in profiles/.  Only the shapes that were profiled have an entry.
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE summaries under profiles/ (not measured in this run)"
 MEASURED_TRAFFIC_BYTES = {
     ("prefill", 4096): (47128 + 28672) * 1024,             # algorithmic 65536 KiB
     ("decode", 16, 32768): (2097572 + 656) * 1024,         # algorithmic 2097152 KiB
@@ -75,7 +79,48 @@ def median(xs):
     return xs[len(xs) // 2]
 
 
-def bench_prefill(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
+SETTLE_MS = 100.0   # launches before any timed batch: the clocks need ~50 ms of load to settle
+BATCHES = 5
+MIN_REPS = 100
+
+
+def settle(torch, step, warmup, min_ms=SETTLE_MS):
+    """At least `warmup` launches and at least `min_ms` of back-to-back launches; returns the ms spent."""
+    t0 = time.perf_counter()
+    i = 0
+    while True:
+        for _ in range(20):
+            step(i)
+            i += 1
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3
+        if ms >= min_ms and i >= warmup:
+            return ms
+
+
+def timed(torch, timer, step, reps):
+    """Median over BATCHES batches of `reps` launches: (event ms per launch, wall ms per launch, all batches)."""
+    ev, wall = [], []
+    for _ in range(BATCHES):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev.append(timer.time_ms(step, reps))
+        torch.cuda.synchronize()
+        wall.append((time.perf_counter() - t0) * 1e3 / reps)
+    return median(ev), median(wall), ev
+
+
+def host_bits(t):
+    import numpy as np
+    return t.detach().cpu().contiguous().view(torch_int16()).numpy().view(np.uint16)
+
+
+def torch_int16():
+    import torch
+    return torch.int16
+
+
+def bench_prefill(ops, torch, timer, S, steps, warmup, H=28, Hkv=4, clock=False):
     g = torch.Generator(device="cuda").manual_seed(1004 + S)
     q = torch.randn(S, H, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
     k = torch.randn(S, Hkv, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
@@ -85,16 +130,37 @@ def bench_prefill(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
     def step(_):
         ops.hip_flash_attn_gqa_layer(out, q, k, v, S, S, 0, H // Hkv, Hkv, 128, DT_BF16)
 
-    for i in range(warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ev_ms = timer.time_ms(step, steps)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    settle_ms = settle(torch, step, warmup)
+    reps = max(steps, MIN_REPS)
+    ev_ms, wall_ms, batches = timed(torch, timer, step, reps)
     flops = 4.0 * H * 128 * S * (S + 1) / 2
-    return {"S": S, "ms_event": ev_ms, "ms_wall": wall_ms, "flops": flops,
-            "tflops": flops / (ev_ms * 1e-3) / 1e12}, (q, k, v, out)
+    r = {"S": S, "ms_event": ev_ms, "ms_wall": wall_ms, "flops": flops, "settle_ms": settle_ms,
+         "launches_per_batch": reps, "batches_us": [b * 1e3 for b in batches],
+         "tflops": flops / (ev_ms * 1e-3) / 1e12}
+    if clock:
+        # shader clock of the first (heaviest) workgroup of one more launch, read inside the kernel
+        probe = torch.zeros(2, dtype=torch.int64, device="cuda")
+        for _ in range(20):
+            step(0)
+        ops.hip_flash_attn_gqa_clocked_layer(out, q, k, v, S, S, 0, H // Hkv, Hkv, 128, DT_BF16, probe)
+        torch.cuda.synchronize()
+        ticks, ref = (int(x) for x in probe.cpu())
+        if ref > 0:
+            r["shader_clock_mhz"] = ticks / ref * 100.0  # the reference counter runs at 100 MHz
+    # accuracy of the timed output: sampled rows against the fp32 oracle (row r of a causal prefill ==
+    # a one-row decode over keys 0..r)
+    import numpy as np
+    from oracle import oracle as orc
+    qb, kb, vb, ob = (host_bits(t) for t in (q, k, v, out))
+    rows = sorted(set([0, 1, 63, 64, 255, 256, S // 2, S - 1] + [int(x) for x in
+                                                               np.random.default_rng(S).integers(0, S, 16)]))
+    worst = 0.0
+    for row in rows:
+        ref = orc.attention_f32(qb[row:row + 1], kb, vb, row + 1, row, DT_BF16)
+        worst = max(worst, float(np.abs(orc.widen(ob[row:row + 1], DT_BF16) - ref).max()))
+    r["max_abs_err"] = worst
+    r["rows_checked"] = len(rows)
+    return r, (q, k, v, out)
 
 
 def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
@@ -122,15 +188,22 @@ def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
         ops.hip_flash_decode_gqa_layer(out, q, ks[0], vs[0], ws, ws_bytes, batch, n, n, H // Hkv,
                                        Hkv, 128, splits, DT_BF16)
 
-    for i in range(warmup):
-        step(i)
+    settle(torch, step, warmup)
+    reps = max(steps, MIN_REPS)
+    cold, _, _ = timed(torch, timer, step, reps)
+    hot_ms, _, _ = timed(torch, timer, hot, reps)
     torch.cuda.synchronize()
-    cold = median([timer.time_ms(step, steps) for _ in range(5)])
-    hot_ms = median([timer.time_ms(hot, steps) for _ in range(3)])
-    torch.cuda.synchronize()
+    # accuracy of the last timed (hot) launch: sequence 0 and the last one against the fp32 oracle
+    import numpy as np
+    from oracle import oracle as orc
+    ob, qb = host_bits(out), host_bits(q)
+    worst = 0.0
+    for b in sorted({0, batch - 1}):
+        ref = orc.attention_f32(qb[b], host_bits(ks[0][b]), host_bits(vs[0][b]), n, n - 1, DT_BF16)
+        worst = max(worst, float(np.abs(orc.widen(ob[b], DT_BF16) - ref).max()))
     return {"batch": batch, "n": n, "splits": splits, "kv_bytes": kv_bytes, "buffers": nbuf,
             "ms_cold": cold, "ms_hot": hot_ms, "gbs_cold": kv_bytes / (cold * 1e-3) / 1e9,
-            "gbs_hot": kv_bytes / (hot_ms * 1e-3) / 1e9}
+            "gbs_hot": kv_bytes / (hot_ms * 1e-3) / 1e9, "max_abs_err": worst}
 
 
 def bench_rope_append(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
@@ -147,12 +220,19 @@ def bench_rope_append(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
     def step(_):
         ops.hip_rope_kv_append_layer(oq, kc, vc, table, q, k, v, 0, S, H, Hkv, 128, True, DT_BF16)
 
-    for i in range(warmup):
-        step(i)
-    torch.cuda.synchronize()
-    ms = median([timer.time_ms(step, steps) for _ in range(3)])
+    settle(torch, step, warmup)
+    ms, _, _ = timed(torch, timer, step, max(steps, MIN_REPS))
     nbytes = 2 * S * 128 * (2 * H + 4 * Hkv) + S * 64 * 8
-    return {"S": S, "ms": ms, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9}
+    # bit-exact against the oracle on the first and last 32 tokens
+    from oracle import oracle as orc
+    tab = table.cpu().numpy()
+    bad = 0
+    for lo in (0, S - 32):
+        sl = slice(lo, lo + 32)
+        bad += int(np.count_nonzero(host_bits(oq[sl]) != orc.rope(host_bits(q[sl]), tab, lo, True, DT_BF16)))
+        bad += int(np.count_nonzero(host_bits(kc[sl]) != orc.rope(host_bits(k[sl]), tab, lo, True, DT_BF16)))
+        bad += int(np.count_nonzero(host_bits(vc[sl]) != host_bits(v[sl])))
+    return {"S": S, "ms": ms, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9, "mismatched_elements": bad}
 
 
 def bench_attention_block(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
@@ -197,13 +277,11 @@ def bench_attention_block(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
         core(i)
         tail(i)
 
-    for i in range(warmup):
-        whole(i)
-    torch.cuda.synchronize()
+    settle(torch, whole, warmup)
     r = {"S": S}
     for name, fn in (("us_total", whole), ("us_qkv_proj", proj_qkv), ("us_rope_attention", core),
                      ("us_o_proj_add", tail)):
-        r[name] = median([timer.time_ms(fn, steps) for _ in range(3)]) * 1e3
+        r[name] = timed(torch, timer, fn, max(steps, 30))[0] * 1e3
     gemm_flops = 2.0 * S * hidden * (2 * hidden + 2 * kvd)
     r["gemm_tflops"] = gemm_flops / ((r["us_qkv_proj"] + r["us_o_proj_add"]) * 1e-6) / 1e12
     return r
@@ -220,7 +298,7 @@ def cpu_baseline(S, H=28, Hkv=4):
     k = orc.round_to(rng.standard_normal((S, Hkv, 128), dtype=np.float32), DT_BF16)
     v = orc.round_to(rng.standard_normal((S, Hkv, 128), dtype=np.float32), DT_BF16)
     flops = 4.0 * H * 128 * S * (S + 1) / 2
-    cores = min(orc.max_threads(), 16)
+    cores = min(orc.max_threads(), 16)  # the box's CPU share for one GPU is 16 threads
     t = time.perf_counter()
     orc.attention_layer(q, k, v, S, 0, DT_BF16, n_threads=cores)
     t_all = time.perf_counter() - t
@@ -230,6 +308,7 @@ def cpu_baseline(S, H=28, Hkv=4):
     return {"value": flops / t_all / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"whole prefill workload (S={S}, H={H}, Hkv={Hkv}, bf16, {flops / 1e9:.1f} GFLOP), "
                       f"layer-style oracle: {t_all:.2f} s on {cores} threads, {t_one:.2f} s on 1 thread",
+            "host_cores_visible": os.cpu_count(),
             "single_thread_value": flops / t_one / 1e12, "seconds_all_cores": t_all,
             "seconds_single_thread": t_one}
 
@@ -265,28 +344,34 @@ def main():
     legs.discard("none")
     extra = {}
 
+    cus, max_mhz, _ = ops.device_props(0)
+    # dense bf16 MFMA: 4 SIMDs x 1024 flop per clock per CU (one 32x32x16 MFMA = 32768 flop in 32 cycles)
+    box_peak_tflops = cus * max_mhz * 1e6 * 4096 / 1e12
+
     # ---- the timed step: prefill at the headline shape ----
     torch.cuda.synchronize()
-    pre, _ = bench_prefill(ops, torch, timer, args.seq, args.steps, args.warmup)
-    log(f"prefill S={args.seq}: {pre['ms_event'] * 1e3:.1f} us  {pre['tflops']:.1f} TFLOP/s")
+    pre, _ = bench_prefill(ops, torch, timer, args.seq, args.steps, args.warmup, clock=True)
+    log(f"prefill S={args.seq}: {pre['ms_event'] * 1e3:.1f} us  {pre['tflops']:.1f} TFLOP/s  "
+        f"max-abs {pre['max_abs_err']:.2e}  shader clock {pre.get('shader_clock_mhz', 0):.0f} MHz")
     if "prefill" in legs:
         others = []
         for S in (1024, 8192):
             if S == args.seq:
                 continue
-            r, _ = bench_prefill(ops, torch, timer, S, max(10, args.steps // 4), max(5, args.warmup // 4))
-            log(f"prefill S={S}: {r['ms_event'] * 1e3:.1f} us  {r['tflops']:.1f} TFLOP/s")
+            r, _ = bench_prefill(ops, torch, timer, S, args.steps, args.warmup)
+            log(f"prefill S={S}: {r['ms_event'] * 1e3:.1f} us  {r['tflops']:.1f} TFLOP/s  max-abs {r['max_abs_err']:.2e}")
             others.append({"S": S, "us": r["ms_event"] * 1e3, "tflops": r["tflops"],
-                           "frac": r["tflops"] / PEAK_BF16_TFLOPS})
+                           "frac": r["tflops"] / PEAK_BF16_TFLOPS, "max_abs_err": r["max_abs_err"]})
         extra["prefill_other"] = others
 
     if "decode" in legs:
         dec = []
         shapes = [tuple(int(x) for x in c.split("x")) for c in args.decode_shapes.split(",") if c]
         for batch, n in shapes:
-            r = bench_decode(ops, torch, timer, batch, n, max(20, args.steps // 2), 10)
+            r = bench_decode(ops, torch, timer, batch, n, args.steps, args.warmup)
             log(f"decode B={batch} n={n} splits={r['splits']}: cold {r['ms_cold'] * 1e3:.1f} us "
-                f"{r['gbs_cold']:.0f} GB/s, hot {r['ms_hot'] * 1e3:.1f} us {r['gbs_hot']:.0f} GB/s")
+                f"{r['gbs_cold']:.0f} GB/s, hot {r['ms_hot'] * 1e3:.1f} us {r['gbs_hot']:.0f} GB/s, "
+                f"max-abs {r['max_abs_err']:.2e}")
             dec.append(r)
             torch.cuda.empty_cache()
         head = dec[0]
@@ -296,22 +381,25 @@ def main():
             "bound": "hbm", "achieved": head["gbs_cold"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
             "frac": head["gbs_cold"] / PEAK_HBM_GBS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(("decode", head["batch"], head["n"])),
+            "traffic_source": TRAFFIC_SOURCE, "max_abs_err": head["max_abs_err"],
             "workload": f"Qwen2.5-32B decode bf16 H=40 Hkv=8 n={head['n']} batch={head['batch']} "
                         f"({head['kv_bytes'] / 2 ** 20:.0f} MiB of K+V per launch, cold)"}
         extra["decode_all"] = [
             {"batch": r["batch"], "n": r["n"], "splits": r["splits"], "us_cold": r["ms_cold"] * 1e3,
              "gbs_cold": r["gbs_cold"], "frac_cold": r["gbs_cold"] / PEAK_HBM_GBS,
-             "us_hot": r["ms_hot"] * 1e3, "gbs_hot": r["gbs_hot"]} for r in dec]
+             "us_hot": r["ms_hot"] * 1e3, "gbs_hot": r["gbs_hot"], "max_abs_err": r["max_abs_err"]} for r in dec]
 
     if "rope" in legs:
-        r = bench_rope_append(ops, torch, timer, args.seq, max(20, args.steps // 2), 10)
+        r = bench_rope_append(ops, torch, timer, args.seq, args.steps, args.warmup)
         log(f"rope+append S={args.seq}: {r['ms'] * 1e3:.1f} us {r['gbs']:.0f} GB/s")
         extra["rope_kv_append"] = {"S": r["S"], "us": r["ms"] * 1e3, "gbs": r["gbs"],
                                    "frac": r["gbs"] / PEAK_HBM_GBS,
-                                   "traffic": MEASURED_TRAFFIC_BYTES.get(("rope", r["S"]))}
+                                   "traffic": MEASURED_TRAFFIC_BYTES.get(("rope", r["S"])),
+                                   "traffic_source": TRAFFIC_SOURCE,
+                                   "mismatched_elements": r["mismatched_elements"]}
 
     if "block" in legs:
-        r = bench_attention_block(ops, torch, timer, args.seq, max(10, args.steps // 8), 3)
+        r = bench_attention_block(ops, torch, timer, args.seq, args.steps // 8, 3)
         log(f"attention block S={args.seq}: {r['us_total']:.0f} us (qkv proj {r['us_qkv_proj']:.0f}, "
             f"rope+attention {r['us_rope_attention']:.0f}, o_proj+add {r['us_o_proj_add']:.0f}; "
             f"GEMMs {r['gemm_tflops']:.0f} TFLOP/s)")
@@ -339,6 +427,11 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": pre["ms_wall"],
+        "settle_ms": pre["settle_ms"],
+        "timing": f"clock-settle phase of >= {SETTLE_MS:.0f} ms of launches, then the median of {BATCHES} batches of "
+                  f"{pre['launches_per_batch']} back-to-back launches between two HIP events on the launch stream",
+        "max_abs_err": pre["max_abs_err"],
+        "max_abs_err_bar": 1e-2,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -350,8 +443,17 @@ def main():
         "roofline": {"bound": "mfma", "achieved": pre["tflops"], "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": pre["tflops"] / PEAK_BF16_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(("prefill", args.seq)),
+                     "traffic_source": TRAFFIC_SOURCE,
                      "kernel": "flash_prefill_kernel<bf16>", "us_per_launch": pre["ms_event"] * 1e3,
-                     "flops_per_launch": pre["flops"]},
+                     "batches_us": pre["batches_us"],
+                     "flops_per_launch": pre["flops"],
+                     "peak_source": "published MI355X dense bf16 MFMA peak (2.5 PFLOP/s, assumes 2.4 GHz)",
+                     "box": {"compute_units": cus, "max_shader_clock_mhz": max_mhz,
+                             "peak_at_max_clock_tflops": box_peak_tflops,
+                             "shader_clock_under_load_mhz": pre.get("shader_clock_mhz"),
+                             "peak_at_clock_under_load_tflops":
+                                 (cus * pre["shader_clock_mhz"] * 1e6 * 4096 / 1e12)
+                                 if pre.get("shader_clock_mhz") else None}},
         "cpu_baseline": cpu,
     }
     line.update(extra)

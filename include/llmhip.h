@@ -60,6 +60,16 @@ int llmhip_flash_attn_opt_prefill(void *out, const void *q, const void *k, const
                                   int m, int n, int offset, int head_num, int head_dim,
                                   int dt, void *stream);
 
+/* Measurement aid with no counterpart in the reference: llmhip_flash_attn_gqa on the prefill
+ * kernel (m * group_size > 16, LLMHIP_ERR_UNSUPPORTED otherwise) that also makes the first
+ * scheduled workgroup store two 64-bit counters at clock_probe (device memory, 16 bytes): the
+ * shader-clock ticks and the ticks of the constant 100 MHz reference clock between its start
+ * and its end.  Their ratio x 100 MHz is the shader clock under this kernel's load, which the
+ * benchmark prints next to the peak it prices against. */
+int llmhip_flash_attn_gqa_clocked(void *out, const void *q, const void *k, const void *v, int m,
+                                  int n, int offset, int group_size, int kv_head_num, int head_dim,
+                                  int dt, void *clock_probe, void *stream);
+
 /* Batched split-KV decode over a contiguous per-sequence KV cache: one query
  * token per sequence, `batch` independent sequences of the same valid length n.
  * q, out: [batch][group_size*kv_head_num][head_dim];
@@ -124,6 +134,9 @@ int llmhip_rope_kv_append(void *out_q, void *k_cache, void *v_cache, const void 
  * aclrtSynchronizeStream (src/llama2_layer_npu.cpp:605-608) and the event
  * calls of src/profiling.cpp:48-78. */
 int llmhip_device_count(void);
+/* Compute units, maximum shader clock (kHz) and memory size of a device (any pointer may be null);
+ * what the benchmark derives the box's own peak from. */
+int llmhip_device_props(int device, int *compute_units, int *max_clock_khz, size_t *total_mem_bytes);
 int llmhip_set_device(int device);
 int llmhip_malloc(void **ptr, size_t bytes);
 int llmhip_free(void *ptr);

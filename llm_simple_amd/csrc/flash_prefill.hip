@@ -51,6 +51,8 @@ struct PrefillParams {
   int sched_mode;  // 0: plain, 1: several XCDs per kv head, 2: several kv heads per XCD
   int sched_a;     // mode 1: XCDs per kv head; mode 2: heads per XCD
   float scale_log2e;
+  // measurement aid, normally null: workgroup 0 stores {shader-clock ticks, 100 MHz ticks} of its lifetime
+  unsigned long long *clock_probe;
 };
 
 // blockIdx -> (query tile, head).  Workgroup ids are dealt round-robin to the 8
@@ -379,6 +381,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tile, head;
   if (!prefill_schedule(p, blockIdx.x, tile, head)) return;
+  unsigned long long clk0 = 0, ref0 = 0;
+  if (p.clock_probe) {
+    clk0 = __builtin_amdgcn_s_memtime();
+    ref0 = __builtin_amdgcn_s_memrealtime();
+  }
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int kvh = head / p.g;
@@ -474,6 +481,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   // every wave is past the last barrier of the loop: nobody reads the K/V tiles any more
   w.store(lds + wave * 32 * kRowBytes, p.out + (size_t)qblk0 * q_row_bytes + (size_t)head * kRowBytes, q_row_bytes,
           p.m - qblk0);
+  if (p.clock_probe && blockIdx.x == 0 && tid == 0) {
+    p.clock_probe[0] = __builtin_amdgcn_s_memtime() - clk0;
+    p.clock_probe[1] = __builtin_amdgcn_s_memrealtime() - ref0;
+  }
 }
 
 template <typename T, int NW>
@@ -527,8 +538,9 @@ static bool prefer_256_rows(int m, int H) {
 
 hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
                                 int n, int offset, int group_size, int kv_head_num, int dt,
-                                hipStream_t stream) {
+                                hipStream_t stream, void *clock_probe) {
   PrefillParams p;
+  p.clock_probe = static_cast<unsigned long long *>(clock_probe);
   p.q = static_cast<const char *>(q);
   p.k = static_cast<const char *>(k);
   p.v = static_cast<const char *>(v);

@@ -100,6 +100,19 @@ int llmhip_flash_attn_opt_prefill(void *out, const void *q, const void *k, const
   return attn_common(out, q, k, v, m, n, offset, 1, head_num, head_dim, dt, stream);
 }
 
+int llmhip_flash_attn_gqa_clocked(void *out, const void *q, const void *k, const void *v, int m,
+                                  int n, int offset, int group_size, int kv_head_num, int head_dim,
+                                  int dt, void *clock_probe, void *stream) {
+  if (!out || !q || !k || !v || !clock_probe) return LLMHIP_ERR_INVALID_ARG;
+  if (m < 1 || n < 1 || offset < 0 || group_size < 1 || kv_head_num < 1 || !dtype_ok(dt))
+    return LLMHIP_ERR_INVALID_ARG;
+  if (head_dim != 128) return LLMHIP_ERR_UNSUPPORTED;
+  if (kv_head_num > 65535 || (long long)group_size * kv_head_num > 65535) return LLMHIP_ERR_UNSUPPORTED;
+  if ((long long)m * group_size <= kMaxDecodeCols) return LLMHIP_ERR_UNSUPPORTED;  // prefill kernel only
+  return from_hip(launch_flash_prefill(out, q, k, v, m, n, offset, group_size, kv_head_num, dt,
+                                       as_stream(stream), clock_probe));
+}
+
 int llmhip_flash_decode_default_splits(int batch, int n, int kv_head_num) {
   if (batch < 1 || n < 1 || kv_head_num < 1) return LLMHIP_ERR_INVALID_ARG;
   return flash_decode_default_splits(batch, n, kv_head_num);
@@ -175,6 +188,16 @@ int llmhip_device_count(void) {
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess) return 0;
   return n;
+}
+int llmhip_device_props(int device, int *compute_units, int *max_clock_khz, size_t *total_mem_bytes) {
+  if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;
+  hipDeviceProp_t prop;
+  hipError_t e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess) return (int)e;
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (max_clock_khz) *max_clock_khz = prop.clockRate;
+  if (total_mem_bytes) *total_mem_bytes = prop.totalGlobalMem;
+  return LLMHIP_OK;
 }
 int llmhip_set_device(int device) {
   if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;

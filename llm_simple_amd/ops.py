@@ -24,6 +24,7 @@ _vp, _i, _i64, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_siz
 SYMBOLS = {
     "llmhip_flash_attn": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_attn_gqa": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "llmhip_flash_attn_gqa_clocked": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "llmhip_flash_attn_opt_prefill": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_gqa": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i64, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
@@ -35,6 +36,7 @@ SYMBOLS = {
     "llmhip_matmul_bias": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "llmhip_add": (_i, [_vp, _vp, _vp, ctypes.c_longlong, _i, _vp]),
     "llmhip_device_count": (_i, []),
+    "llmhip_device_props": (_i, [_i, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_sz)]),
     "llmhip_set_device": (_i, [_i]),
     "llmhip_malloc": (_i, [ctypes.POINTER(_vp), _sz]),
     "llmhip_free": (_i, [_vp]),
@@ -106,6 +108,16 @@ def hip_flash_attn_gqa_layer(output_dev, q_dev, k_dev, v_dev, m, n, offset, grou
     _check(lib.llmhip_flash_attn_gqa(_ptr(output_dev), _ptr(q_dev), _ptr(k_dev), _ptr(v_dev), m,
                                      n, offset, group_size, kv_head_num, head_dim, dt, stream),
            "hip_flash_attn_gqa_layer")
+
+
+def hip_flash_attn_gqa_clocked_layer(output_dev, q_dev, k_dev, v_dev, m, n, offset, group_size,
+                                     kv_head_num, head_dim, dt, clock_probe_dev, stream=0):
+    """hip_flash_attn_gqa_layer on the prefill kernel, which also stores {shader-clock ticks,
+    100 MHz reference ticks} of its first workgroup at clock_probe_dev (two int64)."""
+    _check(lib.llmhip_flash_attn_gqa_clocked(_ptr(output_dev), _ptr(q_dev), _ptr(k_dev), _ptr(v_dev),
+                                             m, n, offset, group_size, kv_head_num, head_dim, dt,
+                                             _ptr(clock_probe_dev), stream),
+           "hip_flash_attn_gqa_clocked_layer")
 
 
 def hip_flash_attn_opt_prefill_layer(output_dev, q_dev, k_dev, v_dev, m, n, offset, head_num,
@@ -180,6 +192,14 @@ def hip_rope_kv_append_layer(output_q_dev, k_cache_dev, v_cache_dev, freqs_cis_d
                                      _ptr(input_v_dev), start_pos, cur_size, n_heads, n_kv_heads,
                                      head_dim, int(bool(is_neox_style)), dt, stream),
            "hip_rope_kv_append_layer")
+
+
+def device_props(device=0):
+    """(compute units, maximum shader clock in MHz, memory bytes) of a device."""
+    cus, khz, mem = _i(0), _i(0), _sz(0)
+    _check(lib.llmhip_device_props(device, ctypes.byref(cus), ctypes.byref(khz), ctypes.byref(mem)),
+           "device_props")
+    return cus.value, khz.value / 1e3, mem.value
 
 
 def _bf16_round_trip(x):

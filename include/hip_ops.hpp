@@ -90,7 +90,7 @@ inline void hip_rope_single_layer(void *output_x_dev, void *freqs_cis_dev, void 
 }
 
 // npu_matmul_nz_layer / npu_matmul_bias_nz_layer (prebuild/npu_ops.h:87-92) with the weight
-// as W[n][k] row-major, and npu_add_layer (prebuild/npu_ops.h:80-81).
+// as W[n][k] row-major, and npu_add_layer (prebuild/npu_ops.h:81-82).
 inline void hip_matmul_layer(void *output_dev, void *lhs_dev, void *rhs_dev, int m, int n, int k,
                              DataType dt, gpuStream_t &stream) {
   CHECK_LLMHIP(llmhip_matmul(output_dev, lhs_dev, rhs_dev, m, n, k, dt, stream));

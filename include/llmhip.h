@@ -89,9 +89,14 @@ int llmhip_flash_decode_gqa(void *out, const void *q, const void *k_cache,
                             int kv_head_num, int head_dim, int num_splits, int dt,
                             void *stream);
 
+/* Workspace size of llmhip_flash_decode_gqa for the same (batch, group_size, kv_head_num, num_splits);
+ * 0 for one split.  num_splits <= 0 gives the size that covers the default split count at any KV
+ * length (at most ceil(256 / (batch * kv_head_num)) splits), so a caller that passes num_splits <= 0
+ * to the decode call can size its workspace once. */
 size_t llmhip_flash_decode_workspace_bytes(int batch, int group_size, int kv_head_num,
                                            int head_dim, int num_splits);
 
+/* The split count the decode call uses for num_splits <= 0: about 256 workgroups in total. */
 int llmhip_flash_decode_default_splits(int batch, int n, int kv_head_num);
 
 /* ------------------------------------------------------------------ */
@@ -176,7 +181,7 @@ int llmhip_matmul(void *out, const void *lhs, const void *weight, int m, int n, 
 int llmhip_matmul_bias(void *out, const void *lhs, const void *weight, const void *bias_f32,
                        int m, int n, int k, int dt, void *stream);
 
-/* Replaces npu_add_layer (prebuild/npu_ops.h:80-81; call site
+/* Replaces npu_add_layer (prebuild/npu_ops.h:81-82; call site
  * src/llama2_layer_npu.cpp:900-901, the residual add after o_proj):
  * out[i] = round_dt(float(lhs[i]) + float(rhs[i])). */
 int llmhip_add(void *out, const void *lhs, const void *rhs, long long total_size, int dt,

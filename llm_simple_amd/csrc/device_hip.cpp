@@ -181,12 +181,15 @@ std::shared_ptr<Tensor> AttentionGPUImpl::Forward(std::shared_ptr<Tensor> q,
   const int cur_size = static_cast<int>(ctx.cur_size);
   const int hidden = n_heads_ * head_dim_;
   if (ctx.cur_pos > static_cast<size_t>(max_seq_len_)) return nullptr;
+  if (!q || !k || !v || !q->data_ptr || !k->data_ptr || !v->data_ptr) return nullptr;
   auto q_emb = Tensor::MakeGPUTensor(static_cast<size_t>(hidden) * cur_size, dtype_);
+  auto out = Tensor::MakeGPUTensor(static_cast<size_t>(hidden) * cur_size, dtype_);
+  if (!q_emb || !out || !q_emb->data_ptr || !out->data_ptr) return nullptr;  // nothing launched yet
+  hip_last_status() = 0;
   hip_rope_kv_append_layer(q_emb->data_ptr, k_cache->data_ptr, v_cache->data_ptr,
                            freq_cis_->data_ptr, q->data_ptr, k->data_ptr, v->data_ptr,
                            static_cast<int>(ctx.prev_pos), cur_size, n_heads_, n_kv_heads_,
                            head_dim_, neox_, dtype_, ctx.gpu_stream);
-  auto out = Tensor::MakeGPUTensor(static_cast<size_t>(hidden) * cur_size, dtype_);
   hip_flash_attn_gqa_layer(out->data_ptr, q_emb->data_ptr, k_cache->data_ptr, v_cache->data_ptr,
                            cur_size, static_cast<int>(ctx.cur_pos), static_cast<int>(ctx.prev_pos),
                            n_heads_ / n_kv_heads_, n_kv_heads_, head_dim_, dtype_, ctx.gpu_stream);
@@ -194,6 +197,8 @@ std::shared_ptr<Tensor> AttentionGPUImpl::Forward(std::shared_ptr<Tensor> q,
   // still read it: drain the stream first, the rule the reference states at
   // src/llama2_layer_npu.cpp:605-608.
   CHECK_LLMHIP(llmhip_stream_sync(ctx.gpu_stream));
+  // a rejected or failed launch leaves `out` unwritten: report it instead of returning garbage
+  if (hip_last_status() != 0) return nullptr;
   return out;
 }
 
@@ -309,7 +314,9 @@ bool MatmulLayerGPUImpl::Init(const void *host_weight, const float *host_bias, s
 
 std::shared_ptr<Tensor> MatmulLayerGPUImpl::Forward(std::shared_ptr<Tensor> input, InferenceCtx &ctx) {
   const int m = static_cast<int>(ctx.cur_size);
+  if (!input || !input->data_ptr) return nullptr;
   auto output = Tensor::MakeGPUTensor(n * ctx.cur_size, dtype_);
+  if (!output || !output->data_ptr) return nullptr;
   char info[96];
   snprintf(info, sizeof(info), "m %d n %zu k %zu", m, n, k);
   APP_PROFILE("MatmulLayer", info, ctx.gpu_stream, ctx.profiler, ctx.is_profiling);
@@ -341,9 +348,18 @@ bool AttentionBlockGPUImpl::Init(const Weights &w, int hidden_dim, int n_heads, 
 std::shared_ptr<Tensor> AttentionBlockGPUImpl::Forward(std::shared_ptr<Tensor> normed,
                                                        std::shared_ptr<Tensor> residual,
                                                        InferenceCtx &ctx) {
+  if (!residual || !residual->data_ptr) return nullptr;
+  hip_last_status() = 0;
   auto q = q_proj.Forward(normed, ctx);
   auto k = k_proj.Forward(normed, ctx);
   auto v = v_proj.Forward(normed, ctx);
+  // Every early return below drains the stream first: the temporaries go back to the pool at scope
+  // exit while launches that read or write them may still be queued.
+  auto bail = [&]() -> std::shared_ptr<Tensor> {
+    CHECK_LLMHIP(llmhip_stream_sync(ctx.gpu_stream));
+    return nullptr;
+  };
+  if (!q || !k || !v || hip_last_status() != 0) return bail();
   std::shared_ptr<Tensor> attn;
   {
     char info[96];
@@ -351,9 +367,10 @@ std::shared_ptr<Tensor> AttentionBlockGPUImpl::Forward(std::shared_ptr<Tensor> n
     APP_PROFILE("RoPE+KVAppend+FlashAttnGQA", info, ctx.gpu_stream, ctx.profiler, ctx.is_profiling);
     attn = attention.Forward(q, k, v, ctx);
   }
-  if (!attn) return nullptr;
+  if (!attn) return bail();
   auto proj = o_proj.Forward(attn, ctx);
   auto out = Tensor::MakeGPUTensor(static_cast<size_t>(hidden_dim_) * ctx.cur_size, dtype_);
+  if (!proj || !out || !out->data_ptr) return bail();
   {
     APP_PROFILE("Add", "attn output + input", ctx.gpu_stream, ctx.profiler, ctx.is_profiling);
     hip_add_layer(out->data_ptr, residual->data_ptr, proj->data_ptr,
@@ -361,6 +378,7 @@ std::shared_ptr<Tensor> AttentionBlockGPUImpl::Forward(std::shared_ptr<Tensor> n
   }
   // temporaries return to the pool at scope exit: drain first (src/llama2_layer_npu.cpp:605-608)
   CHECK_LLMHIP(llmhip_stream_sync(ctx.gpu_stream));
+  if (hip_last_status() != 0) return nullptr;
   return out;
 }
 

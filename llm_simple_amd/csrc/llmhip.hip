@@ -30,8 +30,9 @@ struct StreamScratch {
 std::mutex g_scratch_mu;
 std::map<void *, StreamScratch> g_scratch;
 
-int scratch_for(void *stream, size_t need, void **out) {
-  std::lock_guard<std::mutex> lk(g_scratch_mu);
+// Caller holds g_scratch_mu, and keeps holding it until the launch that uses the buffer is enqueued:
+// a second thread growing the same stream's buffer then cannot free it in between.
+int scratch_for_locked(void *stream, size_t need, void **out) {
   StreamScratch &s = g_scratch[stream];
   if (s.bytes < need) {
     if (s.ptr) {
@@ -67,10 +68,12 @@ int attn_common(void *out, const void *q, const void *k, const void *v, int m, i
     int splits = flash_decode_default_splits(1, n_vis, kv_head_num);
     void *ws = nullptr;
     const size_t need = flash_decode_workspace_bytes(1, m, group_size, kv_head_num, splits);
-    if (need) {
-      int rc = scratch_for(stream, need, &ws);
-      if (rc != LLMHIP_OK) return rc;
-    }
+    if (!need)
+      return from_hip(launch_flash_decode(out, q, k, v, nullptr, 1, m, n_vis, offset, n_vis, group_size,
+                                          kv_head_num, splits, dt, as_stream(stream)));
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    int rc = scratch_for_locked(stream, need, &ws);
+    if (rc != LLMHIP_OK) return rc;
     return from_hip(launch_flash_decode(out, q, k, v, ws, 1, m, n_vis, offset, n_vis,
                                         group_size, kv_head_num, splits, dt,
                                         as_stream(stream)));
@@ -121,6 +124,12 @@ int llmhip_flash_decode_default_splits(int batch, int n, int kv_head_num) {
 size_t llmhip_flash_decode_workspace_bytes(int batch, int group_size, int kv_head_num,
                                            int head_dim, int num_splits) {
   if (batch < 1 || group_size < 1 || kv_head_num < 1 || head_dim != 128) return 0;
+  if (num_splits <= 0) {
+    // the largest count the default rule picks for any KV length: ceil(256 / (batch * kv heads))
+    const long long pairs = (long long)batch * kv_head_num;
+    num_splits = (int)((256 + pairs - 1) / pairs);
+  }
+  if (num_splits > kMaxDecodeSplits) num_splits = kMaxDecodeSplits;
   return flash_decode_workspace_bytes(batch, 1, group_size, kv_head_num, num_splits);
 }
 
@@ -234,7 +243,21 @@ int llmhip_stream_create(void **stream) {
   *stream = s;
   return LLMHIP_OK;
 }
-int llmhip_stream_destroy(void *stream) { return from_hip(hipStreamDestroy(as_stream(stream))); }
+int llmhip_stream_destroy(void *stream) {
+  {
+    // the split-KV scratch kept for this stream goes with it
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    auto it = g_scratch.find(stream);
+    if (it != g_scratch.end()) {
+      if (it->second.ptr) {
+        (void)hipStreamSynchronize(as_stream(stream));
+        (void)hipFree(it->second.ptr);
+      }
+      g_scratch.erase(it);
+    }
+  }
+  return from_hip(hipStreamDestroy(as_stream(stream)));
+}
 int llmhip_stream_sync(void *stream) { return from_hip(hipStreamSynchronize(as_stream(stream))); }
 int llmhip_device_sync(void) { return from_hip(hipDeviceSynchronize()); }
 int llmhip_event_create(void **event) {
@@ -275,6 +298,11 @@ const char *llmhip_error_string(int status) {
 int llmhip_release_internal_workspace(void) {
   std::lock_guard<std::mutex> lk(g_scratch_mu);
   int rc = LLMHIP_OK;
+  if (!g_scratch.empty()) {
+    // queued launches may still use the buffers
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) rc = (int)e;
+  }
   for (auto &kv : g_scratch) {
     if (kv.second.ptr) {
       hipError_t e = hipFree(kv.second.ptr);

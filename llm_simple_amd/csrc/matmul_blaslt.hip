@@ -12,7 +12,7 @@
 // (stored k x n column-major, op T), B = X (k x m column-major, op N), bias along the rows
 // of D (one value per output feature) in the epilogue.
 //
-// Also here: the elementwise residual add (npu_add_layer, prebuild/npu_ops.h:80-81).
+// Also here: the elementwise residual add (npu_add_layer, prebuild/npu_ops.h:81-82).
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 
@@ -33,6 +33,7 @@ struct Plan {
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
   bool ok = false;
+  uint64_t last_use = 0;
 };
 
 // One handle, workspace and plan cache per device.
@@ -40,7 +41,17 @@ struct DeviceBlas {
   hipblasLtHandle_t handle = nullptr;
   void *workspace = nullptr;
   std::map<std::tuple<int, int, int, int, int>, Plan> plans;  // m, n, k, dt, bias
+  uint64_t tick = 0;
 };
+constexpr size_t kMaxPlans = 64;  // per device; the least recently used plan is dropped beyond this
+
+void destroy_plan(Plan &pl) {
+  if (pl.la) hipblasLtMatrixLayoutDestroy(pl.la);
+  if (pl.lb) hipblasLtMatrixLayoutDestroy(pl.lb);
+  if (pl.lc) hipblasLtMatrixLayoutDestroy(pl.lc);
+  if (pl.desc) hipblasLtMatmulDescDestroy(pl.desc);
+  pl = Plan();
+}
 struct Blas {
   std::mutex mu;
   static constexpr size_t kWorkspaceBytes = 64u << 20;
@@ -105,18 +116,25 @@ hipError_t launch_matmul_bias(void *out, const void *lhs, const void *weight, co
       return e;
     }
   }
-  Plan &pl = b.plans[std::make_tuple(m, n, k, dt, bias ? 1 : 0)];
+  const auto key = std::make_tuple(m, n, k, dt, bias ? 1 : 0);
+  if (b.plans.find(key) == b.plans.end() && b.plans.size() >= kMaxPlans) {
+    // every distinct prompt length m makes a plan: keep the cache bounded
+    auto victim = b.plans.begin();
+    for (auto it = b.plans.begin(); it != b.plans.end(); ++it)
+      if (it->second.last_use < victim->second.last_use) victim = it;
+    destroy_plan(victim->second);
+    b.plans.erase(victim);
+  }
+  Plan &pl = b.plans[key];
   if (!pl.ok) {
     e = make_plan(b, pl, m, n, k, dt, bias != nullptr);
     if (e != hipSuccess) {  // nothing half-built stays behind
-      if (pl.la) hipblasLtMatrixLayoutDestroy(pl.la);
-      if (pl.lb) hipblasLtMatrixLayoutDestroy(pl.lb);
-      if (pl.lc) hipblasLtMatrixLayoutDestroy(pl.lc);
-      if (pl.desc) hipblasLtMatmulDescDestroy(pl.desc);
-      pl = Plan();
+      destroy_plan(pl);
+      b.plans.erase(key);
       return e;
     }
   }
+  pl.last_use = ++b.tick;
   if (bias) {
     // the bias pointer is a per-call attribute of the (cached) descriptor; calls are
     // serialised by the mutex above
@@ -137,13 +155,7 @@ void release_matmul_resources() {
   for (auto &dv : all.dev) {
     DeviceBlas &b = dv.second;
     (void)hipSetDevice(dv.first);
-    for (auto &kv : b.plans) {
-      Plan &pl = kv.second;
-      if (pl.la) hipblasLtMatrixLayoutDestroy(pl.la);
-      if (pl.lb) hipblasLtMatrixLayoutDestroy(pl.lb);
-      if (pl.lc) hipblasLtMatrixLayoutDestroy(pl.lc);
-      if (pl.desc) hipblasLtMatmulDescDestroy(pl.desc);
-    }
+    for (auto &kv : b.plans) destroy_plan(kv.second);
     if (b.workspace) (void)hipFree(b.workspace);
     if (b.handle) hipblasLtDestroy(b.handle);
   }

@@ -161,7 +161,7 @@ def hip_matmul_bias_layer(output_dev, lhs_dev, weight_dev, bias_dev, m, n, k, dt
 
 
 def hip_add_layer(output_dev, lhs_dev, rhs_dev, total_size, dt, stream=0):
-    """npu_add_layer (prebuild/npu_ops.h:80-81)."""
+    """npu_add_layer (prebuild/npu_ops.h:81-82)."""
     _check(lib.llmhip_add(_ptr(output_dev), _ptr(lhs_dev), _ptr(rhs_dev), total_size, dt, stream),
            "hip_add_layer")
 

@@ -83,3 +83,24 @@ def test_product_never_touches_the_oracle():
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
     for f in ("llmhip.h", "hip_ops.hpp"):
         assert "oracle" not in open(os.path.join(ROOT, "include", f)).read().lower()
+
+
+def test_default_workspace_size_covers_the_default_split_count():
+    """num_splits <= 0 sizes the workspace for the largest count the default rule can pick, so a
+    caller that lets the decode call choose never gets LLMHIP_ERR_WORKSPACE."""
+    import llm_simple_amd.ops as ops
+    for batch, hkv in ((1, 8), (16, 8), (3, 2), (1, 1), (64, 8)):
+        cover = ops.flash_decode_workspace_bytes(batch, 5, hkv, 128, 0)
+        for n in (1, 100, 4096, 32768, 131072):
+            s = ops.flash_decode_default_splits(batch, n, hkv)
+            assert ops.flash_decode_workspace_bytes(batch, 5, hkv, 128, s) <= cover, (batch, hkv, n)
+
+
+def test_sanitizer_builds_of_oracle_and_device_layer():
+    """Host-only -fsanitize=address,undefined builds: the CPU oracle driven over ragged shapes, and the
+    C++ device layer with its injected allocator backend.  Both targets run what they build."""
+    for sub in ("oracle", os.path.join("tests", "cpp")):
+        r = subprocess.run(["make", "-s", "-C", os.path.join(ROOT, sub), "asan"], capture_output=True,
+                           text=True, timeout=600)
+        assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+        assert "ERROR: AddressSanitizer" not in r.stderr and "runtime error" not in r.stderr, r.stderr[-2000:]

@@ -83,6 +83,6 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None, layer_style=Tr
         # that see few keys land a step or two further away (measured on the kernels over 27 shapes: at most
         # 76 per million beyond TOL-or-2-steps, at most 0.3 per million beyond TOL-or-3-steps)
         off2, off3 = near(2), near(3)
-        assert off2 <= max(2, got.size * 200 // 10 ** 6), f"{off2} of {got.size} elements beyond 2 steps, worst {d16.max()}"
-        assert off3 <= max(1, got.size * 2 // 10 ** 6), f"{off3} of {got.size} elements beyond 3 steps, worst {d16.max()}"
+        assert off2 <= max(4, got.size * 200 // 10 ** 6), f"{off2} of {got.size} elements beyond 2 steps, worst {d16.max()}"
+        assert off3 <= max(2, got.size * 2 // 10 ** 6), f"{off3} of {got.size} elements beyond 3 steps, worst {d16.max()}"
     return e32, float(d16.max())

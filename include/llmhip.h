@@ -99,6 +99,23 @@ size_t llmhip_flash_decode_workspace_bytes(int batch, int group_size, int kv_hea
 /* The split count the decode call uses for num_splits <= 0: about 256 workgroups in total. */
 int llmhip_flash_decode_default_splits(int batch, int n, int kv_head_num);
 
+/* llmhip_flash_decode_gqa for callers that cannot allocate device memory or carry a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments and results as llmhip_flash_decode_gqa without
+ * `workspace`: the split-KV partials go to a fixed array of
+ * llmhip_flash_decode_static_scratch_bytes() (4 MiB) of device memory inside the library, which
+ * every GPU the library runs on holds until the process ends.  The call allocates and frees
+ * nothing.  Limit: batch * kv_head_num * num_splits * 8320 bytes must fit the array (504 slots,
+ * e.g. the default split count for any batch * kv_head_num <= 252); larger requests are rejected
+ * with LLMHIP_ERR_WORKSPACE before anything is launched (one split needs no scratch and always
+ * fits).  All calls on a GPU share the array: calls that overlap on one GPU (different streams,
+ * different threads) race; calls on one stream are ordered and safe. */
+int llmhip_flash_decode_gqa_static(void *out, const void *q, const void *k_cache,
+                                   const void *v_cache, int batch, int n, int64_t kv_seq_stride,
+                                   int group_size, int kv_head_num, int head_dim, int num_splits,
+                                   int dt, void *stream);
+size_t llmhip_flash_decode_static_scratch_bytes(void);
+
 /* ------------------------------------------------------------------ */
 /* rotary embedding and KV-cache append                                */
 /* ------------------------------------------------------------------ */

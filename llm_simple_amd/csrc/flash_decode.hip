@@ -27,6 +27,8 @@
 // two dependent rounds of memory-latency loads in ONE workgroup is longer than a launch.
 // Eight-wave workgroups, half as many, merging pairs of splits through LDS: 4.5 TB/s
 // against 6.0 -- a CU draws about 35 GB/s however many waves ask, so all 256 must stream.)
+#include <atomic>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -382,6 +384,42 @@ hipError_t launch_flash_decode(void *out, const void *q, const void *k, const vo
   else
     hipLaunchKernelGGL(flash_decode_combine_kernel<__bf16>, cgrid, dim3(128), 0, stream, p);
   return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Decode without any allocation: the split-KV partials live in a fixed array in device memory
+// that is part of the library's code object (every GPU the library runs on holds its own copy
+// until the process ends).  In host code the array's name is only a handle for
+// hipGetSymbolAddress: the device address is looked up once per device and that pointer is what
+// the kernels receive, exactly as they receive the caller's workspace in launch_flash_decode.
+// Nothing in the buffer has to start at zero: every (sequence, kv head, split) slot that the
+// combine kernel reads is written by the decode kernel of the same call.  All calls on one GPU
+// share the array, so calls that overlap on one GPU (different streams) race.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[kStaticDecodeScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+}  // namespace
+
+hipError_t launch_flash_decode_static(void *out, const void *q, const void *k, const void *v,
+                                      int batch, int n, int64_t kv_seq_stride, int group_size,
+                                      int kv_head_num, int num_splits, int dt, hipStream_t stream) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    // first call on this device (which is current): each GPU has the array at its own address
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!ptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  return launch_flash_decode(out, q, k, v, ptr, batch, 1, n, n - 1, kv_seq_stride, group_size,
+                             kv_head_num, num_splits, dt, stream);
 }
 
 }  // namespace llmhip

@@ -22,6 +22,13 @@ hipError_t launch_flash_decode(void *out, const void *q, const void *k, const vo
                                int64_t kv_seq_stride, int group_size, int kv_head_num,
                                int num_splits, int dt, hipStream_t stream);
 
+// Same decode with the split-KV partials in a fixed device array of kStaticDecodeScratchBytes inside
+// the library: no allocation, no workspace argument.  The caller checks the size beforehand.
+constexpr size_t kStaticDecodeScratchBytes = 4u << 20;
+hipError_t launch_flash_decode_static(void *out, const void *q, const void *k, const void *v,
+                                      int batch, int n, int64_t kv_seq_stride, int group_size,
+                                      int kv_head_num, int num_splits, int dt, hipStream_t stream);
+
 // q_heads may be 0 (rotate K only) and cache pointers may be null (no append):
 // covers rope, rope_single and the fused rope + KV append.
 hipError_t launch_rope_kv_append(void *out_q, void *out_k, void *out_v, const void *freq_cis,

@@ -153,6 +153,26 @@ int llmhip_flash_decode_gqa(void *out, const void *q, const void *k_cache,
                                       as_stream(stream)));
 }
 
+int llmhip_flash_decode_gqa_static(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                   int batch, int n, int64_t kv_seq_stride, int group_size,
+                                   int kv_head_num, int head_dim, int num_splits, int dt, void *stream) {
+  if (!out || !q || !k_cache || !v_cache) return LLMHIP_ERR_INVALID_ARG;
+  if (batch < 1 || n < 1 || group_size < 1 || kv_head_num < 1 || kv_seq_stride < n)
+    return LLMHIP_ERR_INVALID_ARG;
+  if (!dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
+  if (head_dim != 128 || group_size > kMaxDecodeCols) return LLMHIP_ERR_UNSUPPORTED;
+  if (batch > 65535 || kv_head_num > 65535) return LLMHIP_ERR_UNSUPPORTED;
+  if (num_splits <= 0) num_splits = flash_decode_default_splits(batch, n, kv_head_num);
+  if (num_splits > kMaxDecodeSplits) num_splits = kMaxDecodeSplits;
+  // the fixed array must hold the partials of every (sequence, kv head, split)
+  if (flash_decode_workspace_bytes(batch, 1, group_size, kv_head_num, num_splits) > kStaticDecodeScratchBytes)
+    return LLMHIP_ERR_WORKSPACE;
+  return from_hip(launch_flash_decode_static(out, q, k_cache, v_cache, batch, n, kv_seq_stride, group_size,
+                                             kv_head_num, num_splits, dt, as_stream(stream)));
+}
+
+size_t llmhip_flash_decode_static_scratch_bytes(void) { return kStaticDecodeScratchBytes; }
+
 int llmhip_rope(void *out_q, void *out_k, const void *freq_cis, const void *in_q,
                 const void *in_k, int start_pos, int cur_size, int n_heads, int hidden_dim,
                 int is_neox_style, int dt, void *stream) {
@@ -288,7 +308,9 @@ const char *llmhip_error_string(int status) {
     case LLMHIP_OK: return "ok";
     case LLMHIP_ERR_INVALID_ARG: return "invalid argument";
     case LLMHIP_ERR_UNSUPPORTED: return "unsupported shape (head_dim must be 128)";
-    case LLMHIP_ERR_WORKSPACE: return "workspace missing or too small";
+    case LLMHIP_ERR_WORKSPACE:
+      return "workspace missing or too small (or batch * kv heads * splits beyond the fixed scratch of the "
+             "allocation-free decode)";
     case LLMHIP_ERR_NO_DEVICE: return "no HIP device";
     default: break;
   }

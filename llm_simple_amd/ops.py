@@ -27,6 +27,8 @@ SYMBOLS = {
     "llmhip_flash_attn_gqa_clocked": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "llmhip_flash_attn_opt_prefill": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_gqa": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i64, _i, _i, _i, _i, _i, _vp]),
+    "llmhip_flash_decode_gqa_static": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i64, _i, _i, _i, _i, _i, _vp]),
+    "llmhip_flash_decode_static_scratch_bytes": (_sz, []),
     "llmhip_flash_decode_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "llmhip_flash_decode_default_splits": (_i, [_i, _i, _i]),
     "llmhip_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
@@ -137,6 +139,17 @@ def hip_flash_decode_gqa_layer(output_dev, q_dev, k_cache_dev, v_cache_dev, work
                                        _ptr(v_cache_dev), _ptr(workspace_dev), workspace_bytes,
                                        batch, n, kv_seq_stride, group_size, kv_head_num, head_dim,
                                        num_splits, dt, stream), "hip_flash_decode_gqa_layer")
+
+
+def hip_flash_decode_gqa_static_layer(output_dev, q_dev, k_cache_dev, v_cache_dev, batch, n,
+                                      kv_seq_stride, group_size, kv_head_num, head_dim, num_splits, dt,
+                                      stream=0):
+    """hip_flash_decode_gqa_layer without a workspace: the partials live in a fixed 4 MiB array
+    inside the library and the call allocates nothing."""
+    _check(lib.llmhip_flash_decode_gqa_static(_ptr(output_dev), _ptr(q_dev), _ptr(k_cache_dev),
+                                              _ptr(v_cache_dev), batch, n, kv_seq_stride, group_size,
+                                              kv_head_num, head_dim, num_splits, dt, stream),
+           "hip_flash_decode_gqa_static_layer")
 
 
 def flash_decode_workspace_bytes(batch, group_size, kv_head_num, head_dim, num_splits):

@@ -163,6 +163,32 @@ def bench_prefill(ops, torch, timer, S, steps, warmup, H=28, Hkv=4, clock=False)
     return r, (q, k, v, out)
 
 
+def bench_chunked_prefill(ops, torch, timer, m, n, steps, warmup, H=28, Hkv=4):
+    """A chunk of m new tokens over a cache of n keys (offset = n - m): the prefill kernel with its key range
+    split over workgroups plus the combine launch."""
+    import numpy as np
+    from oracle import oracle as orc
+    g = torch.Generator(device="cuda").manual_seed(1004 + m + n)
+    q = torch.randn(m, H, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+    k = torch.randn(n, Hkv, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+    v = torch.randn(n, Hkv, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+    out = torch.empty_like(q)
+
+    def step(_):
+        ops.hip_flash_attn_gqa_layer(out, q, k, v, m, n, n - m, H // Hkv, Hkv, 128, DT_BF16)
+
+    settle(torch, step, warmup)
+    ev_ms, _, _ = timed(torch, timer, step, max(steps, MIN_REPS))
+    flops = 4.0 * H * 128 * (m * (n - m) + m * (m + 1) / 2)
+    qb, kb, vb, ob = (host_bits(t) for t in (q, k, v, out))
+    worst = 0.0
+    for row in sorted({0, m // 2, m - 1}):
+        ref = orc.attention_f32(qb[row:row + 1], kb, vb, n - m + row + 1, n - m + row, DT_BF16)
+        worst = max(worst, float(np.abs(orc.widen(ob[row:row + 1], DT_BF16) - ref).max()))
+    return {"m": m, "n": n, "H": H, "Hkv": Hkv, "us": ev_ms * 1e3, "tflops": flops / (ev_ms * 1e-3) / 1e12,
+            "kv_gbs": 2.0 * n * Hkv * 256 / (ev_ms * 1e-3) / 1e9, "max_abs_err": worst}
+
+
 def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
     """Cold numbers: successive launches walk over distinct KV buffers whose total
     exceeds 1 GiB, so no launch is served from the 256 MB last-level cache."""
@@ -320,7 +346,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--seq", type=int, default=4096, help="prefill sequence length of the timed step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: prefill,decode,rope,block (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs: prefill,chunked,decode,rope,block (default all)")
     ap.add_argument("--decode-shapes", default="16x32768,1x32768,1x4096,1x16384,16x4096,16x16384",
                     help="comma list of BATCHxKVLEN decode cases; the first one is the headline")
     ap.add_argument("--calib-copy", action="store_true",
@@ -340,7 +366,7 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     timer = HipTimer(ops.lib)
-    legs = set(args.only.split(",")) if args.only else {"prefill", "decode", "rope", "block"}
+    legs = set(args.only.split(",")) if args.only else {"prefill", "chunked", "decode", "rope", "block"}
     legs.discard("none")
     extra = {}
 
@@ -363,6 +389,15 @@ def main():
             others.append({"S": S, "us": r["ms_event"] * 1e3, "tflops": r["tflops"],
                            "frac": r["tflops"] / PEAK_BF16_TFLOPS, "max_abs_err": r["max_abs_err"]})
         extra["prefill_other"] = others
+
+    if "chunked" in legs:
+        rows = []
+        for (m, n, H, Hkv) in ((256, 32768 + 256, 28, 4), (40, 131072, 40, 8)):
+            r = bench_chunked_prefill(ops, torch, timer, m, n, args.steps, args.warmup, H, Hkv)
+            log(f"chunked prefill m={m} n={n} H={H} Hkv={Hkv}: {r['us']:.1f} us  {r['tflops']:.0f} TFLOP/s  "
+                f"K+V {r['kv_gbs']:.0f} GB/s  max-abs {r['max_abs_err']:.2e}")
+            rows.append(r)
+        extra["chunked_prefill"] = rows
 
     if "decode" in legs:
         dec = []

@@ -39,6 +39,7 @@ namespace llmhip {
 constexpr int kTileN = 64;                      // keys per LDS tile
 constexpr int kTileBytes = kTileN * kRowBytes;  // 16 KiB
 constexpr float kLazyLog2 = 8.0f;                // rescale threshold, log2 units
+constexpr int kMaxPrefillSplits = 64;            // key ranges per call (grid.y)
 
 struct PrefillParams {
   const char *q;
@@ -51,38 +52,65 @@ struct PrefillParams {
   int sched_mode;  // 0: plain, 1: several XCDs per kv head, 2: several kv heads per XCD
   int sched_a;     // mode 1: XCDs per kv head; mode 2: heads per XCD
   float scale_log2e;
+  // Key-range split (chunked prefill: few query rows over a long cache).  Split s covers
+  // keys [s*chunk, (s+1)*chunk); with more than one split every workgroup leaves an fp32 partial
+  // (reference maximum, sum, unnormalised O) that prefill_combine_kernel folds.
+  int num_splits, chunk;  // chunk: multiple of 64 keys
+  // Split mode only: the rows of a tile are (token, head-in-group) pairs of ONE kv head, packed
+  // token-major (row index = token * g + head % g), so a chunk shorter than a tile reads K and V of
+  // its kv head once for all g query heads.  blockIdx.x -> (tile, kv head).
+  int pack;
+  float *ws_o;            // [split][m][H][128]
+  float *ws_ml;           // [split][m][H][2]
   // measurement aid, normally null: workgroup 0 stores {shader-clock ticks, 100 MHz ticks} of its lifetime
   unsigned long long *clock_probe;
 };
 
-// blockIdx -> (query tile, head).  Workgroup ids are dealt round-robin to the 8
+// blockIdx -> (query tile, head, key range).  Workgroup ids are dealt round-robin to the 8
 // XCDs by the hardware; heads that share a kv head are kept on the same XCD(s)
 // so that its K/V stay in that XCD's L2, and within an XCD the heaviest (last)
-// query tiles are issued first.
+// query tiles are issued first.  Key ranges (split mode) are the slowest index of an XCD's
+// list, so that every XCD gets the same number of workgroups whatever the head count.
 __device__ __forceinline__ bool prefill_schedule(const PrefillParams &p, int bid, int &tile,
-                                                 int &head) {
+                                                 int &head, int &split) {
   const int T = p.num_q_tiles;
+  if (p.pack) {  // packed rows: items are (key range, tile, kv head)
+    const int per = T * p.Hkv;
+    if (bid >= per * p.num_splits) return false;
+    split = bid / per;
+    const int rem = bid % per;
+    tile = T - 1 - rem / p.Hkv;
+    head = (rem % p.Hkv) * p.g;  // first query head of the kv head
+    return true;
+  }
   if (p.sched_mode == 1) {
     const int X = p.sched_a;
     const int xcd = bid & 7, slot = bid >> 3;
     const int kvh = xcd / X, sub = xcd % X;
-    const int idx = slot * X + sub;
-    if (idx >= p.g * T) return false;
-    tile = T - 1 - idx / p.g;
-    head = kvh * p.g + idx % p.g;
+    const int idx = slot * X + sub, per = p.g * T;
+    if (idx >= per * p.num_splits) return false;
+    split = idx / per;
+    const int rem = idx % per;
+    tile = T - 1 - rem / p.g;
+    head = kvh * p.g + rem % p.g;
     return true;
   }
   if (p.sched_mode == 2) {
     const int hp = p.sched_a;
-    const int xcd = bid & 7, slot = bid >> 3;
-    if (slot >= hp * T) return false;
-    tile = T - 1 - slot / hp;
-    head = xcd * hp + slot % hp;
+    const int xcd = bid & 7, slot = bid >> 3, per = hp * T;
+    if (slot >= per * p.num_splits) return false;
+    split = slot / per;
+    const int rem = slot % per;
+    tile = T - 1 - rem / hp;
+    head = xcd * hp + rem % hp;
     return true;
   }
-  if (bid >= T * p.H) return false;
-  tile = T - 1 - bid / p.H;
-  head = bid % p.H;
+  const int per = T * p.H;
+  if (bid >= per * p.num_splits) return false;
+  split = bid / per;
+  const int rem = bid % per;
+  tile = T - 1 - rem / p.H;
+  head = rem % p.H;
   return true;
 }
 
@@ -311,6 +339,25 @@ template <typename T> struct WaveAttn {
   }
 };
 
+// Partial result of one key range (see PrefillParams::num_splits): this lane's row gets its
+// unnormalised O^T as fp32, and (reference maximum in raw score units, sum) once per lane pair.
+template <typename T>
+__device__ __forceinline__ void store_partial(const WaveAttn<T> &w, float *o_row, float *ml_row, bool row_valid) {
+  const float l_tot = pair_sum(w.l_run);
+  if (!row_valid) return;
+#pragma unroll
+  for (int d = 0; d < 4; ++d)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const f32x4_t v = {w.o[d][4 * i4], w.o[d][4 * i4 + 1], w.o[d][4 * i4 + 2], w.o[d][4 * i4 + 3]};
+      *reinterpret_cast<f32x4_t *>(o_row + 32 * d + 8 * i4 + 4 * w.hh) = v;
+    }
+  if (w.hh == 0) {
+    ml_row[0] = w.m_run;
+    ml_row[1] = l_tot;
+  }
+}
+
 // Global -> LDS tile loader without VGPR staging (global_load_lds_dwordx4: lane l's 16
 // bytes land at the wave-uniform LDS address in M0 + 16*l).  One wave instruction fills four
 // 256-byte rows; the XOR swizzles are realised on the global side: the lane that owns
@@ -379,8 +426,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   constexpr int kVRegion = NSLOT * kTileBytes;
   constexpr int kSplitKK = 3;  // k-steps of S(j+1) issued beside the row-maximum chain
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  int tile, head;
-  if (!prefill_schedule(p, blockIdx.x, tile, head)) return;
+  int tile, head, split;
+  if (!prefill_schedule(p, blockIdx.x, tile, head, split)) return;
   unsigned long long clk0 = 0, ref0 = 0;
   if (p.clock_probe) {
     clk0 = __builtin_amdgcn_s_memtime();
@@ -389,25 +436,50 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int kvh = head / p.g;
+  // Rows of the tile.  Unpacked: rows are tokens of one head.  Packed: row index i stands for token
+  // i / g of head kvh*g + i % g; `rows` counts them.  Everything below works on tokens: qtok is this
+  // lane's token, tok_lo / tok_hi the first / last token of the wave's 32 rows.
+  const int rows = p.pack ? p.m * p.g : p.m;
   const int row0 = tile * BM;
-  const int rows_end = min(p.m, row0 + BM);
-  const int n_vis = min(p.n, rows_end + p.offset);  // keys any row of this tile can see
-  const int J = (n_vis + kTileN - 1) / kTileN;      // 64-key tiles of the workgroup
+  const int rows_end = min(rows, row0 + BM);
+  const int qblk0 = row0 + wave * 32;
+  const int l32_ = lane & 31;
+  const int qidx = min(qblk0 + l32_, rows - 1);
+  const bool row_valid = qblk0 + l32_ < rows;
+  const int qtok = p.pack ? qidx / p.g : qidx;
+  const int qhead = p.pack ? head + qidx % p.g : head;
+  const int tok_lo = p.pack ? qblk0 / p.g : qblk0;
+  const int tok_hi = p.pack ? (min(qblk0 + 31, rows - 1)) / p.g : min(qblk0 + 31, rows - 1);
+  const int tile_tok_end = p.pack ? (rows_end - 1) / p.g + 1 : rows_end;  // one past the tile's last token
+  // This workgroup's key range, seen as a cache of its own: rows [k_lo, k_lo + n_) with the causal
+  // offset shifted accordingly (negative when the range starts past a row's last visible key).
+  const int k_lo = split * p.chunk;
+  const int n_ = min(p.n - k_lo, p.chunk);
+  const int offset_ = p.offset - k_lo;
+  const int n_vis = min(n_, tile_tok_end + offset_);  // keys any row of this tile can see
+  const int J = (n_vis + kTileN - 1) / kTileN;        // 64-key tiles of the workgroup
   const size_t q_row_bytes = (size_t)p.H * kRowBytes;
   const int kv_row_bytes = p.Hkv * kRowBytes;
-  const char *kbase = p.k + (size_t)kvh * kRowBytes;
-  const char *vbase = p.v + (size_t)kvh * kRowBytes;
+  const char *kbase = p.k + (size_t)k_lo * kv_row_bytes + (size_t)kvh * kRowBytes;
+  const char *vbase = p.v + (size_t)k_lo * kv_row_bytes + (size_t)kvh * kRowBytes;
 
   WaveAttn<T> w;
   w.init(lane, kVRegion);
-  const int qblk0 = row0 + wave * 32;
-  const int qrow = qblk0 + w.l32;
-  const int last_row = min(qblk0 + 31, p.m - 1);
-  const int Jw = (qblk0 < p.m) ? min(J, (min(p.n, last_row + p.offset + 1) + kTileN - 1) / kTileN) : 0;
-  w.load_q(p.q + (size_t)min(qrow, p.m - 1) * q_row_bytes + (size_t)head * kRowBytes);
+  const int Jw = (qblk0 < rows) ? max(0, min(J, (min(n_, tok_hi + offset_ + 1) + kTileN - 1) / kTileN)) : 0;
+  float *part_o = nullptr, *part_ml = nullptr;
+  if (p.num_splits > 1) {
+    const size_t slot = ((size_t)split * p.m + qtok) * p.H + qhead;
+    part_o = p.ws_o + slot * kHeadDim;
+    part_ml = p.ws_ml + slot * 2;
+    if (J <= 0) {  // workgroup-uniform: no row of this tile sees a key of this range
+      store_partial(w, part_o, part_ml, row_valid);
+      return;
+    }
+  }
+  w.load_q(p.q + (size_t)qtok * q_row_bytes + (size_t)qhead * kRowBytes);
 
   DirectLoader<NW> ld;
-  ld.init(wave, lane, kv_row_bytes, p.n);
+  ld.init(wave, lane, kv_row_bytes, n_);
   // K runs one tile ahead of V: S(j+1) = K(j+1) Q^T is issued together with the softmax of
   // tile j, so K tile t is fetched SUB+1 iterations and V tile t SUB iterations before use.
 #pragma unroll
@@ -429,8 +501,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
     const int jk = min(j + SUB + 1, J - 1), jv = min(j + SUB, J - 1);
     if (j < Jw) {
       const int key0 = j * kTileN;
-      if ((key0 + kTileN - 1 > qblk0 + p.offset) || (key0 + kTileN > p.n))
-        w.mask(s_cur, key0, qrow, p.offset, p.n);
+      if ((key0 + kTileN - 1 > tok_lo + offset_) || (key0 + kTileN > n_))
+        w.mask(s_cur, key0, qtok, offset_, n_);
       // a burst of loads would stall every wave behind the texture addresser's queue:
       // one load every 16 / PER MFMAs instead
       auto k_hook = [&](int i) {
@@ -479,12 +551,45 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
     }
   }
   // every wave is past the last barrier of the loop: nobody reads the K/V tiles any more
-  w.store(lds + wave * 32 * kRowBytes, p.out + (size_t)qblk0 * q_row_bytes + (size_t)head * kRowBytes, q_row_bytes,
-          p.m - qblk0);
+  if (p.num_splits > 1)  // (packed rows exist in split mode only)
+    store_partial(w, part_o, part_ml, row_valid);
+  else
+    w.store(lds + wave * 32 * kRowBytes, p.out + (size_t)qblk0 * q_row_bytes + (size_t)head * kRowBytes,
+            q_row_bytes, p.m - qblk0);
   if (p.clock_probe && blockIdx.x == 0 && tid == 0) {
     p.clock_probe[0] = __builtin_amdgcn_s_memtime() - clk0;
     p.clock_probe[1] = __builtin_amdgcn_s_memrealtime() - ref0;
   }
+}
+
+// Folds the key-range partials of the output rows with the log-sum-exp rule.  256 threads handle 8
+// (row, head) slots, 32 threads (4 dims each) per slot; grid = ceil(m * H / 8).
+template <typename T>
+__global__ __launch_bounds__(256) void prefill_combine_kernel(PrefillParams p) {
+  using E = Elem<T>;
+  const size_t stride = (size_t)p.m * p.H;  // slots per split
+  const size_t slot = (size_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+  const int d4 = threadIdx.x & 31;
+  if (slot >= stride) return;
+  float M = -INFINITY;
+  for (int s = 0; s < p.num_splits; ++s) M = fmaxf(M, p.ws_ml[(s * stride + slot) * 2]);
+  const float M_use = (M == -INFINITY) ? 0.0f : M;
+  float L = 0.0f;
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int s = 0; s < p.num_splits; ++s) {
+    const float *ml = p.ws_ml + (s * stride + slot) * 2;
+    const float wt = fast_exp2((ml[0] - M_use) * p.scale_log2e);  // exp2(-inf) = 0 for an empty range
+    L += wt * ml[1];
+    const f32x4_t o = *reinterpret_cast<const f32x4_t *>(p.ws_o + (s * stride + slot) * kHeadDim + 4 * d4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] += wt * o[i];
+  }
+  const float inv = (L > 0.0f) ? 1.0f / L : 0.0f;
+  u32x2_t w;
+  w[0] = E::pack2(acc[0] * inv, acc[1] * inv);
+  w[1] = E::pack2(acc[2] * inv, acc[3] * inv);
+  *reinterpret_cast<u32x2_t *>(p.out + slot * kRowBytes + d4 * 8) = w;
 }
 
 template <typename T, int NW>
@@ -493,21 +598,27 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
   constexpr int BM = 32 * NW;
   constexpr int NT = 64 * NW;
   p.num_q_tiles = (p.m + BM - 1) / BM;
+  if (p.pack) p.num_q_tiles = (p.m * p.g + BM - 1) / BM;
   const int T_ = p.num_q_tiles;
   int grid;
-  if (p.Hkv <= 8 && 8 % p.Hkv == 0) {
+  const int S_ = p.num_splits;
+  if (p.pack) {
+    p.sched_mode = 0;
+    p.sched_a = 0;
+    grid = T_ * p.Hkv * S_;
+  } else if (p.Hkv <= 8 && 8 % p.Hkv == 0) {
     p.sched_mode = 1;
     p.sched_a = 8 / p.Hkv;
-    const int per_kvh = p.g * T_;
+    const int per_kvh = p.g * T_ * S_;
     grid = 8 * ((per_kvh + p.sched_a - 1) / p.sched_a);
   } else if (p.Hkv % 8 == 0) {
     p.sched_mode = 2;
     p.sched_a = (p.Hkv / 8) * p.g;
-    grid = 8 * p.sched_a * T_;
+    grid = 8 * p.sched_a * T_ * S_;
   } else {
     p.sched_mode = 0;
     p.sched_a = 0;
-    grid = T_ * p.H;
+    grid = T_ * p.H * S_;
   }
   const size_t lds_bytes = (NW == 8 ? 2 : 1) * 4 * kTileBytes;
   void (*kern)(PrefillParams) = flash_prefill_kernel<T, NW>;
@@ -524,21 +635,83 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
     attr_done.fetch_or(bit, std::memory_order_release);
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds_bytes, stream, p);
+  e = hipGetLastError();
+  if (e != hipSuccess || p.num_splits == 1) return e;
+  hipLaunchKernelGGL(prefill_combine_kernel<T>, dim3((unsigned)(((size_t)p.m * p.H + 7) / 8)), dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 
+// Compute units of the current device (the kernel choice and the key-range split aim at them).
+static int device_compute_units() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int cus = cached[dev].load(std::memory_order_relaxed);
+  if (cus <= 0) {
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    cached[dev].store(cus, std::memory_order_relaxed);
+  }
+  return cus;
+}
+
+// Kernel and key-range split for one call.
 // 256-row workgroups (one per CU) or 128-row ones (two per CU)?  The 256-row kernel has the
 // cheaper step (K/V tiles shared by twice the rows) but coarser work items: with fewer than
 // about one and a half of them per CU the heavy-first list packs badly (the second round is
-// mostly idle) and the 128-row kernel wins.  Measured at H=28, bf16 (128-row / 256-row, us):
-// S=2560 64/73, S=3072 82/88, S=3584 111/107, S=4096 139/131, S=5120 201/194, S=8192 452/438.
-static bool prefer_256_rows(int m, int H) {
-  return (long long)((m + 255) / 256) * H >= 384;
+// mostly idle) and the 128-row kernel wins.  Measured at H=28, bf16, 256 CUs (128-row / 256-row,
+// us): S=2560 64/73, S=3072 82/88, S=3584 111/107, S=4096 139/131, S=5120 201/194, S=8192 452/438.
+// Key-range split: a chunk of few query rows over a long cache (keys >= 8 x rows) makes too few
+// workgroups to fill the chip; its key range is cut so that about one (256-row kernel) or two
+// (128-row kernel) workgroups per CU exist, each with at least 1024 keys.  Square causal prefill is
+// never split: the fp32 partials would cost more HBM traffic than K and V themselves.
+struct PrefillPlan {
+  bool rows256, pack;
+  int num_splits, chunk;
+};
+static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cus) {
+  PrefillPlan pl;
+  const int H = g * Hkv;
+  const long long wg256 = (long long)((m + 255) / 256) * H;
+  pl.rows256 = 2 * wg256 >= 3LL * cus;
+  pl.pack = false;
+  pl.num_splits = 1;
+  pl.chunk = 0x7fffffc0;
+  const long long n_vis = ((long long)m + offset < n) ? (long long)m + offset : n;  // keys the last row sees
+  if (pl.rows256 || n_vis < 8LL * m || n_vis < 2048) return pl;
+  // Split mode.  A chunk shorter than a 128-row tile packs the g query heads of a kv head into the
+  // rows of one tile (K and V of the kv head are then read once, not g times).
+  pl.pack = g > 1 && m < 128;
+  const long long rows = pl.pack ? (long long)m * g : m;  // rows per head (per kv head when packed)
+  const long long groups = pl.pack ? Hkv : H;
+  pl.rows256 = rows >= 192;  // enough rows to use most of a 256-row workgroup
+  const long long wgs = (pl.rows256 ? (rows + 255) / 256 : (rows + 127) / 128) * groups;
+  const long long want_wgs = pl.rows256 ? cus : 2LL * cus;  // one round of workgroups, not one and a bit
+  long long splits = want_wgs / wgs;
+  if (splits > n_vis / 1024) splits = n_vis / 1024;
+  if (splits > kMaxPrefillSplits) splits = kMaxPrefillSplits;
+  if (splits <= 1) {
+    pl.pack = false;
+    pl.rows256 = false;
+    return pl;
+  }
+  long long chunk = (n_vis + splits - 1) / splits;
+  chunk = (chunk + 127) / 128 * 128;
+  pl.chunk = (int)chunk;
+  pl.num_splits = (int)((n_vis + chunk - 1) / chunk);  // no empty trailing range
+  return pl;
+}
+
+size_t flash_prefill_workspace_bytes(int m, int n, int offset, int group_size, int kv_head_num) {
+  const int H = group_size * kv_head_num;
+  const PrefillPlan pl = plan_prefill(m, n, offset, group_size, kv_head_num, device_compute_units());
+  if (pl.num_splits <= 1) return 0;
+  return (size_t)pl.num_splits * m * H * (kHeadDim + 2) * sizeof(float);
 }
 
 hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
                                 int n, int offset, int group_size, int kv_head_num, int dt,
-                                hipStream_t stream, void *clock_probe) {
+                                hipStream_t stream, void *workspace, void *clock_probe) {
   PrefillParams p;
   p.clock_probe = static_cast<unsigned long long *>(clock_probe);
   p.q = static_cast<const char *>(q);
@@ -552,7 +725,19 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
   p.Hkv = kv_head_num;
   p.H = group_size * kv_head_num;
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
-  const bool big = prefer_256_rows(m, p.H);
+  PrefillPlan pl = plan_prefill(m, n, offset, group_size, kv_head_num, device_compute_units());
+  if (pl.num_splits > 1 && !workspace) {  // no scratch offered: run unsplit (and unpacked)
+    pl.num_splits = 1;
+    pl.chunk = 0x7fffffc0;
+    pl.pack = false;
+    pl.rows256 = false;
+  }
+  p.pack = pl.pack ? 1 : 0;
+  p.num_splits = pl.num_splits;
+  p.chunk = pl.chunk;
+  p.ws_o = static_cast<float *>(workspace);
+  p.ws_ml = p.ws_o ? p.ws_o + (size_t)pl.num_splits * m * p.H * kHeadDim : nullptr;
+  const bool big = pl.rows256;
   if (dt == kDtFloat16)
     return big ? launch_prefill_t<_Float16, 8>(p, stream) : launch_prefill_t<_Float16, 4>(p, stream);
   return big ? launch_prefill_t<__bf16, 8>(p, stream) : launch_prefill_t<__bf16, 4>(p, stream);

@@ -7,11 +7,14 @@
 
 namespace llmhip {
 
+// workspace: device memory of flash_prefill_workspace_bytes() bytes (0 = none needed) for the fp32
+// partials of a key-range split; with a null workspace the call runs unsplit.
 // clock_probe: null, or a device pointer to two 64-bit counters that workgroup 0 fills with the
-// shader-clock ticks and the 100 MHz reference ticks of its lifetime (measurement aid).
+// shader-clock ticks and the reference-clock ticks of its lifetime (measurement aid).
+size_t flash_prefill_workspace_bytes(int m, int n, int offset, int group_size, int kv_head_num);
 hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
                                 int n, int offset, int group_size, int kv_head_num, int dt,
-                                hipStream_t stream, void *clock_probe = nullptr);
+                                hipStream_t stream, void *workspace = nullptr, void *clock_probe = nullptr);
 
 // Split-KV decode.  rows = m * group_size <= 16 query rows per kv head.
 size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,

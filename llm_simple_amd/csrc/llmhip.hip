@@ -78,8 +78,18 @@ int attn_common(void *out, const void *q, const void *k, const void *v, int m, i
                                         group_size, kv_head_num, splits, dt,
                                         as_stream(stream)));
   }
+  // a chunk of few rows over a long cache is split over the key range: fp32 partials in the
+  // per-stream scratch
+  const size_t need = flash_prefill_workspace_bytes(m, n, offset, group_size, kv_head_num);
+  if (!need)
+    return from_hip(launch_flash_prefill(out, q, k, v, m, n, offset, group_size, kv_head_num, dt,
+                                         as_stream(stream)));
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  void *ws = nullptr;
+  int rc = scratch_for_locked(stream, need, &ws);
+  if (rc != LLMHIP_OK) return rc;
   return from_hip(launch_flash_prefill(out, q, k, v, m, n, offset, group_size, kv_head_num, dt,
-                                       as_stream(stream)));
+                                       as_stream(stream), ws));
 }
 
 }  // namespace
@@ -113,7 +123,7 @@ int llmhip_flash_attn_gqa_clocked(void *out, const void *q, const void *k, const
   if (kv_head_num > 65535 || (long long)group_size * kv_head_num > 65535) return LLMHIP_ERR_UNSUPPORTED;
   if ((long long)m * group_size <= kMaxDecodeCols) return LLMHIP_ERR_UNSUPPORTED;  // prefill kernel only
   return from_hip(launch_flash_prefill(out, q, k, v, m, n, offset, group_size, kv_head_num, dt,
-                                       as_stream(stream), clock_probe));
+                                       as_stream(stream), nullptr, clock_probe));
 }
 
 int llmhip_flash_decode_default_splits(int batch, int n, int kv_head_num) {

@@ -379,6 +379,38 @@ def test_qwen32b_decode_full_size(batch, n):
         assert np.abs(orc.widen(out, dt) - orc.widen(out_p, dt)).max() <= 2 * 2.0 ** -8
 
 
+CHUNK_CASES = [
+    # (m, n, offset, H, Hkv): few query rows over a long cache -> the key range is split over workgroups
+    (64, 8256, 8192, 28, 4),      # 128-row kernel, every row sees every range
+    (200, 5000, 4800, 28, 4),     # 256-row kernel (m >= 192), ragged last range
+    (256, 33024, 32768, 28, 4),   # the chunked-prefill benchmark shape
+    (100, 9000, 9500, 8, 2),      # n < m + offset: the cache length cuts every row
+    (17, 4099, 4082, 5, 1),       # one 128-row tile, one active wave, odd sizes
+    (40, 20000, 19960, 40, 8),    # Qwen2.5-32B head counts: 200 packed rows per kv head, 256-row kernel
+    (8, 6000, 5992, 28, 4),       # 56 packed rows: one 128-row tile per kv head
+    (20, 3000, 2980, 12, 2),      # 120 packed rows, g = 6
+    (127, 16384, 16257, 14, 2),   # 889 packed rows: four 256-row tiles per kv head, ragged last tile
+    (33, 2500, 2467, 3, 3),       # g = 1: nothing to pack
+]
+
+
+@pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
+@pytest.mark.parametrize("m,n,offset,H,Hkv", CHUNK_CASES)
+def test_chunked_prefill_key_split_vs_oracle(dt, m, n, offset, H, Hkv):
+    """A chunk of m new tokens over a cache of n >> m keys (chunked prefill): the prefill kernel splits the
+    key range over workgroups and folds the fp32 partials (log-sum-exp).  Rows past n are poisoned."""
+    ops = _ops()
+    seed = 500 * m + n + H
+    q = normal_bits(seed, (m, H, 128), dt)
+    k = normal_bits(seed + 1, (n + 5, Hkv, 128), dt)
+    v = normal_bits(seed + 2, (n + 5, Hkv, 128), dt)
+    k[n:] = 0x7FFF
+    v[n:] = 0x7FFF
+    d_out = dev_empty(q.shape)
+    ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), m, n, offset, H // Hkv, Hkv, 128, dt)
+    check_attention(to_host(d_out), q, k, v, n, offset, dt)
+
+
 def test_long_context_131072():
     """A 131072-token cache (the longest context Qwen2.5 advertises) at the 32B head counts: one decode
     step and a 40-token chunk appended at the end (the prefill kernel walking 2048 key tiles), against

@@ -346,7 +346,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--seq", type=int, default=4096, help="prefill sequence length of the timed step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: prefill,chunked,decode,rope,block (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs: ceiling,prefill,chunked,decode,rope,block (default all)")
     ap.add_argument("--decode-shapes", default="16x32768,1x32768,1x4096,1x16384,16x4096,16x16384",
                     help="comma list of BATCHxKVLEN decode cases; the first one is the headline")
     ap.add_argument("--calib-copy", action="store_true",
@@ -366,13 +366,25 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     timer = HipTimer(ops.lib)
-    legs = set(args.only.split(",")) if args.only else {"prefill", "chunked", "decode", "rope", "block"}
+    legs = set(args.only.split(",")) if args.only else {"ceiling", "prefill", "chunked", "decode", "rope", "block"}
     legs.discard("none")
     extra = {}
 
     cus, max_mhz, _ = ops.device_props(0)
     # dense bf16 MFMA: 4 SIMDs x 1024 flop per clock per CU (one 32x32x16 MFMA = 32768 flop in 32 cycles)
     box_peak_tflops = cus * max_mhz * 1e6 * 4096 / 1e12
+
+    # what the matrix pipe of this box sustains on N(0,1) operands: alone, and with the other
+    # instructions of an attention inner loop beside the MFMAs (no memory traffic, no barriers)
+    ceiling = None
+    if "ceiling" in legs:
+        ceiling = {"mfma_only_tflops": ops.probe_mfma_ceiling(0, 150.0),
+                   "attention_mix_tflops": ops.probe_mfma_ceiling(1, 150.0),
+                   "what": "sustained bf16 32x32x16 MFMA rate on N(0,1) operands, 8 waves per CU: the MFMAs alone, "
+                           "and with 6 LDS fragment reads, 13 vector instructions and 4 v_exp_f32 per 4 MFMAs "
+                           "beside them (the prefill loop's mix) -- no memory traffic, barriers or dependences"}
+        log(f"MFMA ceiling on N(0,1) operands: alone {ceiling['mfma_only_tflops']:.0f} TFLOP/s, "
+            f"with the attention instruction mix {ceiling['attention_mix_tflops']:.0f} TFLOP/s")
 
     # ---- the timed step: prefill at the headline shape ----
     torch.cuda.synchronize()
@@ -486,6 +498,9 @@ def main():
                      "box": {"compute_units": cus, "max_shader_clock_mhz": max_mhz,
                              "peak_at_max_clock_tflops": box_peak_tflops,
                              "shader_clock_under_load_mhz": pre.get("shader_clock_mhz"),
+                             "measured_ceiling": ceiling,
+                             "frac_of_attention_mix_ceiling":
+                                 (pre["tflops"] / ceiling["attention_mix_tflops"]) if ceiling else None,
                              "peak_at_clock_under_load_tflops":
                                  (cus * pre["shader_clock_mhz"] * 1e6 * 4096 / 1e12)
                                  if pre.get("shader_clock_mhz") else None}},

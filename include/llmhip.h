@@ -159,6 +159,14 @@ int llmhip_device_count(void);
 /* Compute units, maximum shader clock (kHz) and memory size of a device (any pointer may be null);
  * what the benchmark derives the box's own peak from. */
 int llmhip_device_props(int device, int *compute_units, int *max_clock_khz, size_t *total_mem_bytes);
+/* Measurement aid with no counterpart in the reference: runs, for about target_ms (<= 2000), a loop of
+ * back-to-back bf16 32x32x16 MFMAs on N(0,1) operands on every CU and returns the sustained TFLOP/s.
+ * mix 0: the MFMAs alone (what the matrix pipe sustains at the clock its own power draw allows);
+ * mix 1: the same MFMAs with the LDS fragment reads and vector instructions of a flash-attention
+ * inner loop beside them, no memory traffic, no barriers, no dependences: an upper bound for any
+ * attention kernel with that instruction mix on this machine.  The benchmark prints both next to
+ * the published peak.  Allocates and frees two small device buffers; runs on the default stream. */
+int llmhip_probe_mfma_ceiling(int mix, double target_ms, double *tflops);
 int llmhip_set_device(int device);
 int llmhip_malloc(void **ptr, size_t bytes);
 int llmhip_free(void *ptr);

@@ -47,4 +47,8 @@ void release_matmul_resources();
 hipError_t launch_add(void *out, const void *lhs, const void *rhs, size_t total, int dt,
                       hipStream_t stream);
 
+// Measurement aid (ceiling_probe.hip): sustained MFMA TFLOP/s of this GPU on N(0,1) bf16 operands,
+// mix 0 = MFMAs alone, mix 1 = MFMAs with the LDS reads and vector instructions of an attention loop.
+hipError_t run_mfma_ceiling(int mix, double target_ms, double *tflops_out);
+
 }  // namespace llmhip

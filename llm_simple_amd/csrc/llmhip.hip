@@ -238,6 +238,11 @@ int llmhip_device_props(int device, int *compute_units, int *max_clock_khz, size
   if (total_mem_bytes) *total_mem_bytes = prop.totalGlobalMem;
   return LLMHIP_OK;
 }
+int llmhip_probe_mfma_ceiling(int mix, double target_ms, double *tflops) {
+  if (!tflops || (mix != 0 && mix != 1) || target_ms < 0.0 || target_ms > 2000.0) return LLMHIP_ERR_INVALID_ARG;
+  if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;
+  return from_hip(run_mfma_ceiling(mix, target_ms, tflops));
+}
 int llmhip_set_device(int device) {
   if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;
   return from_hip(hipSetDevice(device));

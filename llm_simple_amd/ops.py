@@ -39,6 +39,7 @@ SYMBOLS = {
     "llmhip_add": (_i, [_vp, _vp, _vp, ctypes.c_longlong, _i, _vp]),
     "llmhip_device_count": (_i, []),
     "llmhip_device_props": (_i, [_i, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_sz)]),
+    "llmhip_probe_mfma_ceiling": (_i, [_i, ctypes.c_double, ctypes.POINTER(ctypes.c_double)]),
     "llmhip_set_device": (_i, [_i]),
     "llmhip_malloc": (_i, [ctypes.POINTER(_vp), _sz]),
     "llmhip_free": (_i, [_vp]),
@@ -213,6 +214,14 @@ def device_props(device=0):
     _check(lib.llmhip_device_props(device, ctypes.byref(cus), ctypes.byref(khz), ctypes.byref(mem)),
            "device_props")
     return cus.value, khz.value / 1e3, mem.value
+
+
+def probe_mfma_ceiling(mix, target_ms=60.0):
+    """Sustained bf16 MFMA TFLOP/s on N(0,1) operands: mix 0 = MFMAs alone, mix 1 = with the LDS reads and
+    vector instructions of an attention inner loop beside them."""
+    t = ctypes.c_double(0.0)
+    _check(lib.llmhip_probe_mfma_ceiling(mix, float(target_ms), ctypes.byref(t)), "probe_mfma_ceiling")
+    return t.value
 
 
 def _bf16_round_trip(x):

@@ -255,65 +255,81 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
   }
 }
 
-// grid (rows, Hkv, batch), 128 threads: folds the splits of one output row with
-// the log-sum-exp rule.  The per-split (max, sum) pairs are read once, in
-// parallel, into LDS; thread d then accumulates its column with independent
-// loads in flight.
+// Folds the splits of one output row (one query row of one head) with the log-sum-exp rule.
+// grid (rows, Hkv, batch), 256 threads = 8 groups of 32: group sg takes splits sg, sg+8, ... (four
+// dims per thread, all of a thread's loads issued before any is used), then the 8 groups are merged
+// through LDS.  With few splits the surplus groups have nothing to load.
 constexpr int kMaxSplits = 256;
 
 template <typename T>
-__global__ __launch_bounds__(128) void flash_decode_combine_kernel(DecodeParams p) {
+__global__ __launch_bounds__(256) void flash_decode_combine_kernel(DecodeParams p) {
   using E = Elem<T>;
-  __shared__ float w_s[kMaxSplits];
-  __shared__ float red[4];
+  __shared__ float red_m[8], red_l[8];
+  __shared__ f32x4_t red_o[8][32];
   const int c = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-  const int d = threadIdx.x;
+  const int sg = threadIdx.x >> 5, d4 = threadIdx.x & 31;
   const int S = p.num_splits;
   const size_t base = ((size_t)b * p.Hkv + kvh) * S;
-  // pass 1: this thread owns splits d and d + 128
-  float m0 = -INFINITY, m1 = -INFINITY, l0 = 0.0f, l1 = 0.0f;
-  if (d < S) {
-    m0 = p.ws_ml[((base + d) * kDecCols + c) * 2];
-    l0 = p.ws_ml[((base + d) * kDecCols + c) * 2 + 1];
-  }
-  if (d + 128 < S) {
-    m1 = p.ws_ml[((base + d + 128) * kDecCols + c) * 2];
-    l1 = p.ws_ml[((base + d + 128) * kDecCols + c) * 2 + 1];
-  }
-  float M = fmaxf(m0, m1);
+  const float *ml = p.ws_ml + (base * kDecCols + c) * 2;
+  const float *src = p.ws_o + (base * kDecCols + c) * kHeadDim + 4 * d4;
+  const size_t ml_stride = (size_t)kDecCols * 2, o_stride = (size_t)kDecCols * kHeadDim;
+  float M = -INFINITY, L = 0.0f;
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = sg; s0 < S; s0 += 32) {  // rounds of up to 4 splits per thread
+    float mv[4], lv[4];
+    f32x4_t ov[4];
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
-  if ((d & 63) == 0) red[d >> 6] = M;
+    for (int j = 0; j < 4; ++j) {
+      const int s = min(s0 + 8 * j, S - 1);
+      mv[j] = ml[s * ml_stride];
+      lv[j] = ml[s * ml_stride + 1];
+      ov[j] = *reinterpret_cast<const f32x4_t *>(src + s * o_stride);
+    }
+    float Mn = M;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (s0 + 8 * j < S) Mn = fmaxf(Mn, mv[j]);
+    const float M_use = (Mn == -INFINITY) ? 0.0f : Mn;
+    const float resc = fast_exp2(M - M_use);  // 0 on the first round (M = -inf)
+    L *= resc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] *= resc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float wt = (s0 + 8 * j < S) ? fast_exp2(mv[j] - M_use) : 0.0f;
+      L += wt * lv[j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] += wt * ov[j][i];
+    }
+    M = Mn;
+  }
+  if (d4 == 0) {
+    red_m[sg] = M;
+    red_l[sg] = L;
+  }
+  red_o[sg][d4] = acc;
   __syncthreads();
-  M = fmaxf(red[0], red[1]);
-  const float M_use = (M == -INFINITY) ? 0.0f : M;
-  const float w0 = fast_exp2(m0 - M_use), w1 = fast_exp2(m1 - M_use);
-  if (d < S) w_s[d] = w0;
-  if (d + 128 < S) w_s[d + 128] = w1;
-  float L = w0 * l0 + w1 * l1;
+  if (sg != 0) return;
+  float Mt = -INFINITY;
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
-  if ((d & 63) == 0) red[2 + (d >> 6)] = L;
-  __syncthreads();
-  L = red[2] + red[3];
-  // pass 2: weighted sum of the partial outputs
-  const float *src = p.ws_o + (base * kDecCols + c) * kHeadDim + d;
-  const size_t stride = (size_t)kDecCols * kHeadDim;
-  float acc = 0.0f;
-  int s = 0;
-  for (; s + 8 <= S; s += 8) {
-    float x[8];
+  for (int g8 = 0; g8 < 8; ++g8) Mt = fmaxf(Mt, red_m[g8]);
+  const float Mt_use = (Mt == -INFINITY) ? 0.0f : Mt;
+  float Lt = 0.0f;
+  f32x4_t tot = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) x[j] = src[(size_t)(s + j) * stride];
+  for (int g8 = 0; g8 < 8; ++g8) {
+    const float wt = fast_exp2(red_m[g8] - Mt_use);  // 0 for a group without splits (-inf)
+    Lt += wt * red_l[g8];
+    const f32x4_t o = red_o[g8][d4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc += w_s[s + j] * x[j];
+    for (int i = 0; i < 4; ++i) tot[i] += wt * o[i];
   }
-  for (; s < S; ++s) acc += w_s[s] * src[(size_t)s * stride];
-  const float inv = (L > 0.0f) ? 1.0f / L : 0.0f;
+  const float inv = (Lt > 0.0f) ? 1.0f / Lt : 0.0f;
   const int r = c / p.g, hq = c % p.g;
-  uint16_t *op = reinterpret_cast<uint16_t *>(
-      p.out + (((size_t)b * p.m + r) * p.H + kvh * p.g + hq) * kRowBytes);
-  op[d] = E::round(acc * inv);
+  u32x2_t w;
+  w[0] = E::pack2(tot[0] * inv, tot[1] * inv);
+  w[1] = E::pack2(tot[2] * inv, tot[3] * inv);
+  *reinterpret_cast<u32x2_t *>(p.out + (((size_t)b * p.m + r) * p.H + kvh * p.g + hq) * kRowBytes + d4 * 8) = w;
 }
 
 static int decode_chunk(int n, int num_splits) {
@@ -380,9 +396,9 @@ hipError_t launch_flash_decode(void *out, const void *q, const void *k, const vo
   if (e != hipSuccess || p.num_splits == 1) return e;
   dim3 cgrid(p.rows, kv_head_num, batch);
   if (dt == kDtFloat16)
-    hipLaunchKernelGGL(flash_decode_combine_kernel<_Float16>, cgrid, dim3(128), 0, stream, p);
+    hipLaunchKernelGGL(flash_decode_combine_kernel<_Float16>, cgrid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL(flash_decode_combine_kernel<__bf16>, cgrid, dim3(128), 0, stream, p);
+    hipLaunchKernelGGL(flash_decode_combine_kernel<__bf16>, cgrid, dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -143,18 +143,21 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// State of one wave: 32 query rows (one per lane pair), fp32 O^T accumulators.
-template <typename T> struct WaveAttn {
+// State of one wave: 32 query rows (one per lane pair), fp32 O^T accumulators.  KB = 32-key blocks
+// of every 64-key tile that the wave works on: 2 normally; 1 when two waves share the rows and
+// each takes one half of every tile (short sequences: halves the serial MFMA chain of a wave).
+template <typename T, int KB = 2> struct WaveAttn {
   using E = Elem<T>;
   f32x16_t o[4];       // O^T: d block x (16 d rows of this lane)
-  u32x4_t pf[2][2];    // P^T packed as B operand: key block x k-step
+  u32x4_t pf[KB][2];   // P^T packed as B operand: key block x k-step
   u32x4_t qf[8];       // Q^T fragments (B operand), loaded once
   float m_run, l_run;  // running max (raw score units) and sum of this lane's keys
   int lane, l32, hh, g16, li;
   int k_addr[8];  // LDS byte offset of this lane's K fragment kk in tile slot 0, key block 0
   int v_addr[4];  // same for the V^T fragment of d block d (k-step 0, low half)
 
-  __device__ __forceinline__ void init(int lane_, int v_region) {
+  // kb0: first 32-key block of a tile this wave works on (0, or 1 for the second wave of a pair)
+  __device__ __forceinline__ void init(int lane_, int v_region, int kb0 = 0) {
     lane = lane_;
     l32 = lane & 31;
     hh = lane >> 5;
@@ -171,13 +174,13 @@ template <typename T> struct WaveAttn {
     // compiler from recomputing them (it otherwise spends ~50 VALU instructions per tile).
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) {
-      k_addr[kk] = k_swizzle_off(l32, 2 * kk + hh);
+      k_addr[kk] = k_swizzle_off(l32, 2 * kk + hh) + kb0 * 32 * kRowBytes;
       asm volatile("" : "+v"(k_addr[kk]));
     }
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       const int gran = d * 4 + (g16 & 1) * 2 + ((li & 3) >> 1);
-      v_addr[d] = v_region + v_swizzle_off(4 * hh + (li >> 2), gran) + (li & 1) * 8;
+      v_addr[d] = v_region + v_swizzle_off(4 * hh + (li >> 2), gran) + (li & 1) * 8 + kb0 * 32 * kRowBytes;
       asm volatile("" : "+v"(v_addr[d]));
     }
   }
@@ -196,15 +199,15 @@ template <typename T> struct WaveAttn {
   struct NoHook {
     __device__ __forceinline__ void operator()(int) const {}
   };
-  // S^T = K Q^T for the 64 keys of the K tile at byte offset `koff` of the LDS segment.
+  // S^T = K Q^T for the wave's keys of the K tile at byte offset `koff` of the LDS segment.
   // The fragments of step kk+1 are requested before the MFMAs of step kk.  hook(i) runs
-  // after MFMA i (0..15): the callers spread their global loads over the MFMA stream with it.
+  // after MFMA i (0..8*KB-1): the callers spread their global loads over the MFMA stream with it.
   template <int KK0 = 0, int KK1 = 8, typename Hook = NoHook>
-  __device__ __forceinline__ void qk(const char *lds, int koff, f32x16_t (&s)[2], Hook hook = Hook()) {
+  __device__ __forceinline__ void qk(const char *lds, int koff, f32x16_t (&s)[KB], Hook hook = Hook()) {
 #pragma unroll
     for (int kk = KK0; kk < KK1; ++kk) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+      for (int kb = 0; kb < KB; ++kb) {
         const u32x4_t kf = lds_read_b128(lds, k_addr[kk] + koff + kb * 32 * kRowBytes);
         if (kk == 0) {
           f32x16_t z;
@@ -214,7 +217,7 @@ template <typename T> struct WaveAttn {
         } else {
           s[kb] = E::mfma32(kf, qf[kk], s[kb]);
         }
-        hook(kk * 2 + kb);
+        hook(kk * KB + kb);
       }
     }
   }
@@ -225,7 +228,7 @@ template <typename T> struct WaveAttn {
   template <typename Hook = NoHook>
   __device__ __forceinline__ void pv(const char *lds, int voff, Hook hook = Hook()) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
       for (int ks2 = 0; ks2 < 2; ++ks2) {
 #pragma unroll
@@ -240,10 +243,11 @@ template <typename T> struct WaveAttn {
       }
   }
 
-  // Causal / length mask of one tile of scores (only called for tiles that can be cut).
-  __device__ __forceinline__ void mask(f32x16_t (&s)[2], int key0, int qrow, int offset, int n) {
+  // Causal / length mask of one tile of scores (only called for tiles that can be cut); key0 =
+  // first key of the wave's part of the tile.
+  __device__ __forceinline__ void mask(f32x16_t (&s)[KB], int key0, int qrow, int offset, int n) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = key0 + kb * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
@@ -253,10 +257,10 @@ template <typename T> struct WaveAttn {
 
   // P = exp2(s*c + neg_ms) rounded to T and packed as the B operand; returns this lane's sum
   // of the rounded values.
-  __device__ __forceinline__ float probabilities(const f32x16_t (&s)[2], float c, float neg_ms) {
+  __device__ __forceinline__ float probabilities(const f32x16_t (&s)[KB], float c, float neg_ms) {
     float ps0 = 0.0f, ps1 = 0.0f;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
       for (int ks2 = 0; ks2 < 2; ++ks2) {
         u32x4_t w;
@@ -287,12 +291,18 @@ template <typename T> struct WaveAttn {
   // in log2 units (probabilities then stay below 2^kLazyLog2, harmless in fp32 sums and in
   // the 16-bit P operand); a -inf reference always moves.  O and l are rescaled only then,
   // which after the first tiles is rare.  Returns the additive term of the exponent.
-  __device__ __forceinline__ float row_max(const f32x16_t (&s)[2], float scale_log2e) {
+  __device__ __forceinline__ float row_max(const f32x16_t (&s)[KB], float scale_log2e) {
     float m0 = -INFINITY, m1 = -INFINITY;  // two chains: half the dependent latency
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      m0 = fmaxf(m0, s[0][i]);
-      m1 = fmaxf(m1, s[1][i]);
+      if (KB == 2) {
+        m0 = fmaxf(m0, s[0][i]);
+        m1 = fmaxf(m1, s[KB - 1][i]);
+      } else if (i & 1) {
+        m1 = fmaxf(m1, s[0][i]);
+      } else {
+        m0 = fmaxf(m0, s[0][i]);
+      }
     }
     const float mloc = pair_max(fmaxf(m0, m1));
     const bool move = mloc > m_run + kLazyLog2 / scale_log2e;
@@ -308,6 +318,30 @@ template <typename T> struct WaveAttn {
       m_run = m_new;
     }
     return -((m_run == -INFINITY) ? 0.0f : m_run) * scale_log2e;
+  }
+
+  // Two waves that shared the rows (KB == 1): the second writes its state to LDS lane by lane
+  // (66 floats per lane, stride 64 floats between a lane's values: conflict-free), the first folds
+  // it into its own.  The reference maxima are uniform over a lane pair in both waves.
+  __device__ __forceinline__ void export_state(float *lds_pair) const {
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) lds_pair[(d * 16 + i) * 64 + lane] = o[d][i];
+    lds_pair[64 * 64 + lane] = m_run;
+    lds_pair[65 * 64 + lane] = l_run;
+  }
+  __device__ __forceinline__ void import_state(const float *lds_pair, float scale_log2e) {
+    const float m_b = lds_pair[64 * 64 + lane], l_b = lds_pair[65 * 64 + lane];
+    const float m_new = fmaxf(m_run, m_b);
+    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+    const float fa = fast_exp2((m_run - m_use) * scale_log2e), fb = fast_exp2((m_b - m_use) * scale_log2e);
+    l_run = l_run * fa + l_b * fb;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[d][i] = o[d][i] * fa + lds_pair[(d * 16 + i) * 64 + lane] * fb;
+    m_run = m_new;
   }
 
   // out[row][head][0..127] = O^T / l, rounded once.  The lane layout of O^T (a lane holds 4
@@ -341,8 +375,8 @@ template <typename T> struct WaveAttn {
 
 // Partial result of one key range (see PrefillParams::num_splits): this lane's row gets its
 // unnormalised O^T as fp32, and (reference maximum in raw score units, sum) once per lane pair.
-template <typename T>
-__device__ __forceinline__ void store_partial(const WaveAttn<T> &w, float *o_row, float *ml_row, bool row_valid) {
+template <typename T, int KB>
+__device__ __forceinline__ void store_partial(const WaveAttn<T, KB> &w, float *o_row, float *ml_row, bool row_valid) {
   const float l_tot = pair_sum(w.l_run);
   if (!row_valid) return;
 #pragma unroll
@@ -413,17 +447,21 @@ template <int NW> struct DirectLoader {
 // Every wave runs S(j+1) = K Q^T, the softmax of tile j and P(j).V(j) as one instruction
 // stream (the compiler interleaves the softmax VALU work with the MFMAs); the tile loads
 // are spread over that stream.  NW = 4: two workgroups per CU (small problems); NW = 8:
-// one workgroup per CU, K/V tiles shared by 256 rows.
+// one workgroup per CU, K/V tiles shared by 256 rows.  KB = 1 (with NW = 8): 128 rows, every row
+// block worked on by two waves that each take one 32-key half of every tile and are merged
+// through LDS at the end -- for sequences so short that there is at most about one 128-row
+// workgroup per CU, where the serial MFMA chain of a wave is what the launch waits for.
 // ---------------------------------------------------------------------------
-template <typename T, int NW>
+template <typename T, int NW, int KB>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel(PrefillParams p) {
   // SUB tiles of 64 keys per stage and per barrier: with one workgroup per CU (NW = 8) a stage
   // holds 128 keys, which halves the number of times the waves are forced in step.
   // LDS: K tiles of both stages [2*SUB][16 KiB], then the V tiles likewise; tile t sits in
   // slot t % (2*SUB) of each region, so every fragment address is a per-lane register plus a
   // constant below 64 KiB.
-  constexpr int BM = 32 * NW, PER = 16 / NW, SUB = NW == 8 ? 2 : 1, NSLOT = 2 * SUB;
+  constexpr int BM = 16 * NW * KB, RB = BM / 32, PER = 16 / NW, SUB = NW == 8 ? 2 : 1, NSLOT = 2 * SUB;
   constexpr int kVRegion = NSLOT * kTileBytes;
+  constexpr int kWaveKeys = 32 * KB;  // keys of a tile per wave
   constexpr int kSplitKK = 3;  // k-steps of S(j+1) issued beside the row-maximum chain
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tile, head, split;
@@ -442,7 +480,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   const int rows = p.pack ? p.m * p.g : p.m;
   const int row0 = tile * BM;
   const int rows_end = min(rows, row0 + BM);
-  const int qblk0 = row0 + wave * 32;
+  const int rb = wave % RB, kpar = wave / RB;  // row block; which half of every tile (KB == 1)
+  const int kw0 = (KB == 1) ? 32 * kpar : 0;   // first key of the wave's part of a tile
+  const int qblk0 = row0 + rb * 32;
   const int l32_ = lane & 31;
   const int qidx = min(qblk0 + l32_, rows - 1);
   const bool row_valid = qblk0 + l32_ < rows;
@@ -463,9 +503,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   const char *kbase = p.k + (size_t)k_lo * kv_row_bytes + (size_t)kvh * kRowBytes;
   const char *vbase = p.v + (size_t)k_lo * kv_row_bytes + (size_t)kvh * kRowBytes;
 
-  WaveAttn<T> w;
-  w.init(lane, kVRegion);
-  const int Jw = (qblk0 < rows) ? max(0, min(J, (min(n_, tok_hi + offset_ + 1) + kTileN - 1) / kTileN)) : 0;
+  WaveAttn<T, KB> w;
+  w.init(lane, kVRegion, (KB == 1) ? kpar : 0);
+  // tiles in which this wave's keys hold at least one visible key
+  const int Jw = (qblk0 < rows) ? max(0, min(J, (min(n_, tok_hi + offset_ + 1) - kw0 + kTileN - 1) / kTileN)) : 0;
   float *part_o = nullptr, *part_ml = nullptr;
   if (p.num_splits > 1) {
     const size_t slot = ((size_t)split * p.m + qtok) * p.H + qhead;
@@ -493,22 +534,22 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   ld.wait_all();
   lds_barrier();
 
-  f32x16_t sa[2], sb[2];  // scores of the current / the next tile, roles alternate
+  f32x16_t sa[KB], sb[KB];  // scores of the current / the next tile, roles alternate
   if (Jw > 0) w.qk(lds, 0, sa);
 
-  auto tile_step = [&](int j, int slot, f32x16_t (&s_cur)[2], f32x16_t (&s_nxt)[2]) {
+  auto tile_step = [&](int j, int slot, f32x16_t (&s_cur)[KB], f32x16_t (&s_nxt)[KB]) {
     const int kslot = (slot + SUB + 1) % NSLOT, vslot = (slot + SUB) % NSLOT;  // fetched now
     const int jk = min(j + SUB + 1, J - 1), jv = min(j + SUB, J - 1);
     if (j < Jw) {
-      const int key0 = j * kTileN;
-      if ((key0 + kTileN - 1 > tok_lo + offset_) || (key0 + kTileN > n_))
+      const int key0 = j * kTileN + kw0;
+      if ((key0 + kWaveKeys - 1 > tok_lo + offset_) || (key0 + kWaveKeys > n_))
         w.mask(s_cur, key0, qtok, offset_, n_);
       // a burst of loads would stall every wave behind the texture addresser's queue:
-      // one load every 16 / PER MFMAs instead
+      // one load every 8 * KB / PER MFMAs instead
       auto k_hook = [&](int i) {
 #pragma unroll
         for (int r = 0; r < PER; ++r)
-          if (i == (16 / PER) * r + 1) ld.template issue<false>(kbase, jk, kslot * kTileBytes, r);
+          if (i == (8 * KB / PER) * r + 1) ld.template issue<false>(kbase, jk, kslot * kTileBytes, r);
       };
       // The MFMAs of S(j+1) overlap the softmax of tile j: the first ones run beside the row
       // maximum chain, the rest -- and the MFMAs of P.V -- beside the exponentials.  (For the
@@ -522,7 +563,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
       w.pv(lds, slot * kTileBytes, [&](int i) {
 #pragma unroll
         for (int r = 0; r < PER; ++r)
-          if (i == (16 / PER) * r + 1)
+          if (i == (8 * KB / PER) * r + 1)
             ld.template issue<true>(vbase, jv, kVRegion + vslot * kTileBytes, r);
       });
     } else {
@@ -551,10 +592,19 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
     }
   }
   // every wave is past the last barrier of the loop: nobody reads the K/V tiles any more
+  if (KB == 1) {
+    // the two waves of a row block: the second hands its state over (behind the RB output
+    // staging regions of 8 KiB), the first folds it in and stores
+    float *pair = reinterpret_cast<float *>(lds + RB * 32 * kRowBytes) + (size_t)rb * 66 * 64;
+    if (kpar == 1) w.export_state(pair);
+    __syncthreads();
+    if (kpar == 1) return;
+    w.import_state(pair, p.scale_log2e);
+  }
   if (p.num_splits > 1)  // (packed rows exist in split mode only)
     store_partial(w, part_o, part_ml, row_valid);
   else
-    w.store(lds + wave * 32 * kRowBytes, p.out + (size_t)qblk0 * q_row_bytes + (size_t)head * kRowBytes,
+    w.store(lds + rb * 32 * kRowBytes, p.out + (size_t)qblk0 * q_row_bytes + (size_t)head * kRowBytes,
             q_row_bytes, p.m - qblk0);
   if (p.clock_probe && blockIdx.x == 0 && tid == 0) {
     p.clock_probe[0] = __builtin_amdgcn_s_memtime() - clk0;
@@ -592,10 +642,10 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(PrefillParams p) {
   *reinterpret_cast<u32x2_t *>(p.out + slot * kRowBytes + d4 * 8) = w;
 }
 
-template <typename T, int NW>
+template <typename T, int NW, int KB = 2>
 static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) {
   PrefillParams p = p0;
-  constexpr int BM = 32 * NW;
+  constexpr int BM = 16 * NW * KB;
   constexpr int NT = 64 * NW;
   p.num_q_tiles = (p.m + BM - 1) / BM;
   if (p.pack) p.num_q_tiles = (p.m * p.g + BM - 1) / BM;
@@ -621,7 +671,7 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
     grid = T_ * p.H * S_;
   }
   const size_t lds_bytes = (NW == 8 ? 2 : 1) * 4 * kTileBytes;
-  void (*kern)(PrefillParams) = flash_prefill_kernel<T, NW>;
+  void (*kern)(PrefillParams) = flash_prefill_kernel<T, NW, KB>;
   // the opt-in for more than 64 KiB of dynamic LDS is per device: once per device and kernel
   static std::atomic<uint64_t> attr_done{0};
   int dev = 0;
@@ -667,6 +717,7 @@ static int device_compute_units() {
 // never split: the fp32 partials would cost more HBM traffic than K and V themselves.
 struct PrefillPlan {
   bool rows256, pack;
+  bool pair;  // 128-row workgroups of 8 waves, two waves per row block (short sequences)
   int num_splits, chunk;
 };
 static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cus) {
@@ -675,10 +726,16 @@ static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cu
   const long long wg256 = (long long)((m + 255) / 256) * H;
   pl.rows256 = 2 * wg256 >= 3LL * cus;
   pl.pack = false;
+  // at most about one 128-row workgroup per CU: the launch waits for the serial chain of the wave
+  // with the most keys, so two waves share every row block (measured at H=28, bf16: S=1024 22.6 us
+  // with 4-wave workgroups)
+  pl.pair = !pl.rows256 && 4 * (long long)((m + 127) / 128) * H <= 5LL * cus;
   pl.num_splits = 1;
   pl.chunk = 0x7fffffc0;
   const long long n_vis = ((long long)m + offset < n) ? (long long)m + offset : n;  // keys the last row sees
+  if (n_vis < 256) pl.pair = false;
   if (pl.rows256 || n_vis < 8LL * m || n_vis < 2048) return pl;
+  pl.pair = false;
   // Split mode.  A chunk shorter than a 128-row tile packs the g query heads of a kv head into the
   // rows of one tile (K and V of the kv head are then read once, not g times).
   pl.pack = g > 1 && m < 128;
@@ -693,6 +750,7 @@ static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cu
   if (splits <= 1) {
     pl.pack = false;
     pl.rows256 = false;
+    pl.pair = 4 * (long long)((m + 127) / 128) * H <= 5LL * cus;
     return pl;
   }
   long long chunk = (n_vis + splits - 1) / splits;
@@ -737,10 +795,10 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
   p.chunk = pl.chunk;
   p.ws_o = static_cast<float *>(workspace);
   p.ws_ml = p.ws_o ? p.ws_o + (size_t)pl.num_splits * m * p.H * kHeadDim : nullptr;
-  const bool big = pl.rows256;
-  if (dt == kDtFloat16)
-    return big ? launch_prefill_t<_Float16, 8>(p, stream) : launch_prefill_t<_Float16, 4>(p, stream);
-  return big ? launch_prefill_t<__bf16, 8>(p, stream) : launch_prefill_t<__bf16, 4>(p, stream);
+  const bool f16 = dt == kDtFloat16;
+  if (pl.rows256) return f16 ? launch_prefill_t<_Float16, 8>(p, stream) : launch_prefill_t<__bf16, 8>(p, stream);
+  if (pl.pair) return f16 ? launch_prefill_t<_Float16, 8, 1>(p, stream) : launch_prefill_t<__bf16, 8, 1>(p, stream);
+  return f16 ? launch_prefill_t<_Float16, 4>(p, stream) : launch_prefill_t<__bf16, 4>(p, stream);
 }
 
 }  // namespace llmhip

@@ -349,6 +349,8 @@ def main():
     ap.add_argument("--only", default="", help="comma list of legs: ceiling,prefill,chunked,decode,rope,block (default all)")
     ap.add_argument("--decode-shapes", default="16x32768,1x32768,1x4096,1x16384,16x4096,16x16384",
                     help="comma list of BATCHxKVLEN decode cases; the first one is the headline")
+    ap.add_argument("--chunk-shapes", default="256x33024x28x4,40x131072x40x8",
+                    help="comma list of MxNxHxHKV chunked-prefill cases (M new tokens over a cache of N keys)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times (known traffic: 1 GiB read + "
                          "1 GiB written per launch) so that FETCH_SIZE / WRITE_SIZE of a rocprofv3 --pmc run "
@@ -404,7 +406,7 @@ def main():
 
     if "chunked" in legs:
         rows = []
-        for (m, n, H, Hkv) in ((256, 32768 + 256, 28, 4), (40, 131072, 40, 8)):
+        for (m, n, H, Hkv) in [tuple(int(x) for x in c.split("x")) for c in args.chunk_shapes.split(",") if c]:
             r = bench_chunked_prefill(ops, torch, timer, m, n, args.steps, args.warmup, H, Hkv)
             log(f"chunked prefill m={m} n={n} H={H} Hkv={Hkv}: {r['us']:.1f} us  {r['tflops']:.0f} TFLOP/s  "
                 f"K+V {r['kv_gbs']:.0f} GB/s  max-abs {r['max_abs_err']:.2e}")

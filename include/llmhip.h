@@ -60,6 +60,16 @@ int llmhip_flash_attn_opt_prefill(void *out, const void *q, const void *k, const
                                   int m, int n, int offset, int head_num, int head_dim,
                                   int dt, void *stream);
 
+/* How many bytes of the library's per-stream scratch buffer a llmhip_flash_attn* call with these
+ * arguments uses (head_num of the MHA entry points = kv_head_num with group_size 1): the fp32
+ * partials of the split-KV decode kernel (m * group_size <= 16) or of a key-range split of the
+ * prefill kernel (a chunk of few rows over a cache at least 8 times longer); 0 for ordinary
+ * prefill shapes.  The buffer is allocated on the first call that needs it on a stream (at least
+ * 4 MiB), grows when a later call needs more, and is freed by llmhip_stream_destroy or
+ * llmhip_release_internal_workspace: a caller that must not see an allocation later warms the
+ * stream up with its largest shape. */
+size_t llmhip_flash_attn_scratch_bytes(int m, int n, int offset, int group_size, int kv_head_num);
+
 /* Measurement aid with no counterpart in the reference: llmhip_flash_attn_gqa on the prefill
  * kernel (m * group_size > 16, LLMHIP_ERR_UNSUPPORTED otherwise) that also makes the first
  * scheduled workgroup store two 64-bit counters at clock_probe (device memory, 16 bytes): the

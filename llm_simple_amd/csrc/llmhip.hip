@@ -126,6 +126,16 @@ int llmhip_flash_attn_gqa_clocked(void *out, const void *q, const void *k, const
                                        as_stream(stream), nullptr, clock_probe));
 }
 
+size_t llmhip_flash_attn_scratch_bytes(int m, int n, int offset, int group_size, int kv_head_num) {
+  if (m < 1 || n < 1 || offset < 0 || group_size < 1 || kv_head_num < 1) return 0;
+  if ((long long)m * group_size <= kMaxDecodeCols) {
+    const int n_vis = (n < m + offset) ? n : m + offset;
+    return flash_decode_workspace_bytes(1, m, group_size, kv_head_num,
+                                        flash_decode_default_splits(1, n_vis, kv_head_num));
+  }
+  return flash_prefill_workspace_bytes(m, n, offset, group_size, kv_head_num);
+}
+
 int llmhip_flash_decode_default_splits(int batch, int n, int kv_head_num) {
   if (batch < 1 || n < 1 || kv_head_num < 1) return LLMHIP_ERR_INVALID_ARG;
   return flash_decode_default_splits(batch, n, kv_head_num);

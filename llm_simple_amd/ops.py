@@ -24,6 +24,7 @@ _vp, _i, _i64, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_siz
 SYMBOLS = {
     "llmhip_flash_attn": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_attn_gqa": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "llmhip_flash_attn_scratch_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "llmhip_flash_attn_gqa_clocked": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "llmhip_flash_attn_opt_prefill": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_gqa": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i64, _i, _i, _i, _i, _i, _vp]),

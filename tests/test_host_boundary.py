@@ -104,3 +104,21 @@ def test_sanitizer_builds_of_oracle_and_device_layer():
                            text=True, timeout=600)
         assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
         assert "ERROR: AddressSanitizer" not in r.stderr and "runtime error" not in r.stderr, r.stderr[-2000:]
+
+
+def test_internal_scratch_size_of_the_reference_signature_calls():
+    """Which llmhip_flash_attn* shapes take scratch from the per-stream buffer, and how much: none for square
+    causal prefill, split-KV partials for decode-like shapes, key-range partials for a short chunk over a
+    long cache (sized for the default 256 compute units when no GPU is visible)."""
+    import llm_simple_amd.ops as ops
+    f = ops.lib.llmhip_flash_attn_scratch_bytes
+    for S in (256, 1024, 4096, 8192):
+        assert f(S, S, 0, 7, 4) == 0            # Qwen2.5-7B prefill
+    assert f(256, 256, 0, 1, 32) == 0           # Llama2-7B prefill
+    assert f(1, 512, 511, 1, 32) == 32 * 4 * 16 * 130 * 4     # decode: 32 kv heads x 4 splits of 128 keys
+    assert f(1, 32768, 32767, 5, 8) == ops.flash_decode_workspace_bytes(1, 5, 8, 128, 32)
+    chunk = f(256, 33024, 32768, 7, 4)          # chunked prefill: 9 key ranges x 256 rows x 28 heads
+    assert chunk == 9 * 256 * 28 * 130 * 4
+    packed = f(40, 131072, 131032, 5, 8)        # 200 packed rows per kv head, 32 key ranges
+    assert packed == 32 * 40 * 40 * 130 * 4
+    assert f(0, 10, 0, 1, 1) == 0 and f(4, 0, 0, 1, 1) == 0   # invalid arguments

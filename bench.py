@@ -41,10 +41,12 @@ DT_BF16 = 5
 # figures are in profiles/.  Only the shapes that were profiled have an entry.
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE summaries under profiles/ (not measured in this run)"
 MEASURED_TRAFFIC_BYTES = {
-    ("prefill", 4096): (47128 + 28672) * 1024,             # algorithmic 65536 KiB
+    ("prefill", 4096): (47179 + 28672) * 1024,             # algorithmic 65536 KiB
     ("decode", 16, 32768): (2097572 + 656) * 1024,         # algorithmic 2097152 KiB
     ("decode", 1, 32768): (131250 + 656) * 1024,           # algorithmic 131072 KiB
-    ("rope", 4096): (40530 + 36864) * 1024,                # algorithmic 75776 KiB
+    ("rope", 4096): (40527 + 36864) * 1024,                # algorithmic 75776 KiB
+    ("chunked", 256, 33024): (136014 + 33557 + 33339 + 1792) * 1024,   # prefill kernel + combine
+    ("chunked", 40, 131072): (524998 + 26241 + 26437 + 400) * 1024,
 }
 
 
@@ -186,6 +188,7 @@ def bench_chunked_prefill(ops, torch, timer, m, n, steps, warmup, H=28, Hkv=4):
         ref = orc.attention_f32(qb[row:row + 1], kb, vb, n - m + row + 1, n - m + row, DT_BF16)
         worst = max(worst, float(np.abs(orc.widen(ob[row:row + 1], DT_BF16) - ref).max()))
     return {"m": m, "n": n, "H": H, "Hkv": Hkv, "us": ev_ms * 1e3, "tflops": flops / (ev_ms * 1e-3) / 1e12,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(("chunked", m, n)), "traffic_source": TRAFFIC_SOURCE,
             "kv_gbs": 2.0 * n * Hkv * 256 / (ev_ms * 1e-3) / 1e9, "max_abs_err": worst}
 
 

@@ -726,10 +726,11 @@ static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cu
   const long long wg256 = (long long)((m + 255) / 256) * H;
   pl.rows256 = 2 * wg256 >= 3LL * cus;
   pl.pack = false;
-  // at most about one 128-row workgroup per CU: the launch waits for the serial chain of the wave
-  // with the most keys, so two waves share every row block (measured at H=28, bf16: S=1024 22.6 us
-  // with 4-wave workgroups)
-  pl.pair = !pl.rows256 && 4 * (long long)((m + 127) / 128) * H <= 5LL * cus;
+  // up to two 128-row workgroups per CU: the launch waits for the serial chain of the waves with
+  // the most keys, so two waves share every row block (measured at H=28, bf16, 256 CUs, 4-wave /
+  // paired 8-wave workgroups, us: S=1024 22.6/20.2, S=1536 32.8/27.9, S=2048 45.6/42.1,
+  // S=2560 60.8/64.6, S=3072 76.3/86.0)
+  pl.pair = !pl.rows256 && (long long)((m + 127) / 128) * H <= 2LL * cus;
   pl.num_splits = 1;
   pl.chunk = 0x7fffffc0;
   const long long n_vis = ((long long)m + offset < n) ? (long long)m + offset : n;  // keys the last row sees
@@ -750,7 +751,7 @@ static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cu
   if (splits <= 1) {
     pl.pack = false;
     pl.rows256 = false;
-    pl.pair = 4 * (long long)((m + 127) / 128) * H <= 5LL * cus;
+    pl.pair = (long long)((m + 127) / 128) * H <= 2LL * cus;
     return pl;
   }
   long long chunk = (n_vis + splits - 1) / splits;

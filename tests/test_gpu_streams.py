@@ -1,0 +1,87 @@
+"""Stream behaviour of the operators through the C ABI: they run on the stream they are given (results on a
+created stream equal the default-stream results bit for bit), and the launches that allocate nothing can be
+captured in a HIP graph and replayed (every replay checked against the eager result, with eager work and
+synchronisations between the replays)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from helpers import DT_BFLOAT16, DT_FLOAT16, dev_empty, f32_dev, normal_bits, to_dev, to_host
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _chain(ops, stream, d_table, d_q, d_k, d_v, d_kc, d_vc, d_qe, d_o, d_q1, d_o1, m, H, Hkv, dt):
+    """rope + append of m tokens at row 0, causal attention over them, then one decode step over the cache."""
+    ops.hip_rope_kv_append_layer(d_qe, d_kc, d_vc, d_table, d_q, d_k, d_v, 0, m, H, Hkv, 128, True, dt, stream)
+    ops.hip_flash_attn_gqa_layer(d_o, d_qe, d_kc, d_vc, m, m, 0, H // Hkv, Hkv, 128, dt, stream)
+    ops.hip_flash_decode_gqa_static_layer(d_o1, d_q1, d_kc, d_vc, 1, m, m, H // Hkv, Hkv, 128, 0, dt, stream)
+
+
+@pytest.mark.parametrize("dt", [DT_BFLOAT16, DT_FLOAT16])
+def test_created_stream_equals_default_stream(dt):
+    import torch
+    import llm_simple_amd.ops as ops
+    m, H, Hkv = 300, 12, 2
+    table = f32_dev(orc.init_freq_cis(128, 512, 1e6, dt))
+    q, k, v = (to_dev(normal_bits(s, (m, h, 128), dt)) for s, h in ((1, H), (2, Hkv), (3, Hkv)))
+    q1 = to_dev(normal_bits(4, (1, H, 128), dt))
+    outs = []
+    s = ctypes.c_void_p()
+    assert ops.lib.llmhip_stream_create(ctypes.byref(s)) == 0
+    try:
+        for stream in (0, s.value):
+            kc, vc = dev_empty((512, Hkv, 128)).zero_(), dev_empty((512, Hkv, 128)).zero_()
+            qe, o, o1 = dev_empty((m, H, 128)), dev_empty((m, H, 128)), dev_empty((1, H, 128))
+            torch.cuda.synchronize()
+            _chain(ops, stream, table, q, k, v, kc, vc, qe, o, q1, o1, m, H, Hkv, dt)
+            # also the reference-signature decode (per-stream scratch of the library)
+            o2 = dev_empty((1, H, 128))
+            ops.hip_flash_attn_gqa_layer(o2, q1, kc, vc, 1, m, m - 1, H // Hkv, Hkv, 128, dt, stream)
+            assert ops.lib.llmhip_stream_sync(stream) == 0
+            outs.append([to_host(t).copy() for t in (qe, kc, vc, o, o1, o2)])
+        for a, b in zip(*outs):
+            assert np.array_equal(a, b)
+        assert np.array_equal(outs[0][4], outs[0][5])  # static decode == reference-signature decode
+    finally:
+        assert ops.lib.llmhip_stream_destroy(s) == 0
+
+
+def test_graph_capture_and_replay():
+    import torch
+    import llm_simple_amd.ops as ops
+    dt, m, H, Hkv = DT_BFLOAT16, 200, 28, 4
+    table = f32_dev(orc.init_freq_cis(128, 256, 1e6, dt))
+    mk = lambda seed, h, rows=m: to_dev(normal_bits(seed, (rows, h, 128), dt))
+    d_q, d_k, d_v, d_q1 = mk(10, H), mk(11, Hkv), mk(12, Hkv), mk(13, H, 1)
+    kc, vc = dev_empty((256, Hkv, 128)).zero_(), dev_empty((256, Hkv, 128)).zero_()
+    qe, o, o1 = dev_empty((m, H, 128)), dev_empty((m, H, 128)), dev_empty((1, H, 128))
+    torch.cuda.synchronize()
+    # eager once first (module load, LDS attribute of the kernels): nothing of that belongs in a capture
+    _chain(ops, 0, table, d_q, d_k, d_v, kc, vc, qe, o, d_q1, o1, m, H, Hkv, dt)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _chain(ops, torch.cuda.current_stream().cuda_stream, table, d_q, d_k, d_v, kc, vc, qe, o, d_q1, o1, m, H,
+               Hkv, dt)
+    for rep in range(4):
+        # new inputs in the captured buffers, eager result into separate outputs
+        for t, seed, h, rows in ((d_q, 100, H, m), (d_k, 200, Hkv, m), (d_v, 300, Hkv, m), (d_q1, 400, H, 1)):
+            t.copy_(to_dev(normal_bits(seed + rep, (rows, h, 128), dt)))
+        kc2, vc2 = dev_empty((256, Hkv, 128)).zero_(), dev_empty((256, Hkv, 128)).zero_()
+        qe2, o2, o12 = dev_empty((m, H, 128)), dev_empty((m, H, 128)), dev_empty((1, H, 128))
+        _chain(ops, 0, table, d_q, d_k, d_v, kc2, vc2, qe2, o2, d_q1, o12, m, H, Hkv, dt)
+        torch.cuda.synchronize()
+        want = [to_host(t).copy() for t in (qe2, kc2, vc2, o2, o12)]
+        for t in (qe, o, o1):
+            t.fill_(0x7FFF)  # stale results must not survive
+        kc.zero_()
+        vc.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [to_host(t).copy() for t in (qe, kc, vc, o, o1)]
+        for a, b in zip(got, want):
+            assert np.array_equal(a, b), f"replay {rep}"

@@ -19,16 +19,23 @@
 // moves lazily, so O is rarely rescaled.  Accumulation is fp32; out =
 // O / l rounded once; l sums the ROUNDED probabilities (what P.V used).
 //
-// flash_prefill_kernel<T, NW>: NW waves share the K/V tiles of 32*NW query rows.
-// NW = 8 (one workgroup per CU) once there are about 1.5 such workgroups per CU, NW = 4
-// (two workgroups per CU) for smaller problems.  Tiles travel global -> LDS without
-// VGPR staging (global_load_lds_dwordx4), spread over the MFMA stream.  The loop is
-// software pipelined inside a wave: the MFMAs of S(j+1) are issued beside the softmax
-// of tile j (the first ones beside the row-maximum chain, the rest, together with the
+// flash_prefill_kernel<T, NW, KB>: NW waves share the K/V tiles of 16*NW*KB query rows.
+// NW = 8, KB = 2 (256 rows, one workgroup per CU) once there are about 1.5 such workgroups per CU;
+// NW = 4, KB = 2 (128 rows, two workgroups per CU) below that; NW = 8, KB = 1 (128 rows, two waves
+// per row block, each taking one 32-key half of every tile) up to two 128-row workgroups per CU.
+// Tiles travel global -> LDS without VGPR staging (global_load_lds_dwordx4), spread over the MFMA
+// stream.  The loop is software pipelined inside a wave: the MFMAs of S(j+1) are issued beside the
+// softmax of tile j (the first ones beside the row-maximum chain, the rest, together with the
 // MFMAs of P(j).V(j), beside the exponentials), so K is fetched one tile ahead of V.
 // Every LDS fragment address is a loop-invariant register plus an immediate, and a
 // tile load is a scalar base plus a loop-invariant lane offset: the loop spends its
 // vector ALU instructions on the softmax only.
+//
+// A chunk of few query rows over a long cache (chunked prefill) has its key range split over
+// workgroups: each leaves an fp32 partial (reference maximum, sum, unnormalised O) and
+// prefill_combine_kernel folds them; a chunk shorter than a tile packs the query heads of a kv
+// head into the rows of one tile.  plan_prefill decides all of this from the shape and the
+// device's CU count.
 #include <atomic>
 
 #include "common.hpp"
@@ -39,7 +46,7 @@ namespace llmhip {
 constexpr int kTileN = 64;                      // keys per LDS tile
 constexpr int kTileBytes = kTileN * kRowBytes;  // 16 KiB
 constexpr float kLazyLog2 = 8.0f;                // rescale threshold, log2 units
-constexpr int kMaxPrefillSplits = 64;            // key ranges per call (grid.y)
+constexpr int kMaxPrefillSplits = 64;            // key ranges per call
 
 struct PrefillParams {
   const char *q;
@@ -58,7 +65,7 @@ struct PrefillParams {
   int num_splits, chunk;  // chunk: multiple of 64 keys
   // Split mode only: the rows of a tile are (token, head-in-group) pairs of ONE kv head, packed
   // token-major (row index = token * g + head % g), so a chunk shorter than a tile reads K and V of
-  // its kv head once for all g query heads.  blockIdx.x -> (tile, kv head).
+  // its kv head once for all g query heads.
   int pack;
   float *ws_o;            // [split][m][H][128]
   float *ws_ml;           // [split][m][H][2]

@@ -427,3 +427,30 @@ def test_long_context_131072():
         d_out = dev_empty(q.shape)
         ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), dk, dv, m, n, n - m, H // Hkv, Hkv, 128, dt)
         check_attention(to_host(d_out), q, k, v, n, n - m, dt)
+
+
+def test_flash_decode_random_shapes():
+    """Seeded sweep of the batched decode entry point: batch, KV length, allocated rows per sequence, group
+    size and kv heads drawn at random (group sizes up to the 16 columns of the kernel), default splits."""
+    import torch
+    ops = _ops()
+    rng = np.random.default_rng(20250101)
+    for i in range(24):
+        dt = DT_BFLOAT16 if i % 2 else DT_FLOAT16
+        batch = int(rng.integers(1, 6))
+        n = int(rng.choice([1, 2, 31, 32, 33, 127, 128, 129, int(rng.integers(130, 3000))]))
+        stride = n + int(rng.choice([0, 1, 17]))
+        g = int(rng.choice([1, 2, 3, 5, 7, 8, 16]))
+        Hkv = int(rng.choice([1, 2, 3, 8]))
+        H = g * Hkv
+        q = normal_bits(9000 + i, (batch, 1, H, 128), dt)
+        k = normal_bits(9100 + i, (batch, stride, Hkv, 128), dt)
+        v = normal_bits(9200 + i, (batch, stride, Hkv, 128), dt)
+        k[:, n:] = 0x7FFF
+        v[:, n:] = 0x7FFF
+        wsb = ops.flash_decode_workspace_bytes(batch, g, Hkv, 128, 0)
+        ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
+        d_out = dev_empty((batch, 1, H, 128))
+        ops.hip_flash_decode_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), ws, wsb, batch, n, stride, g, Hkv,
+                                       128, 0, dt)
+        check_attention(to_host(d_out), q, k, v, n, n - 1, dt, batch=True)

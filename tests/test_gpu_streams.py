@@ -85,3 +85,27 @@ def test_graph_capture_and_replay():
         got = [to_host(t).copy() for t in (qe, kc, vc, o, o1)]
         for a, b in zip(got, want):
             assert np.array_equal(a, b), f"replay {rep}"
+
+
+def test_measurement_aids():
+    """The clocked prefill entry returns the same output as the plain one and plausible counters; the MFMA
+    ceiling probe returns a rate between a tenth of the published peak and the peak."""
+    import torch
+    import llm_simple_amd.ops as ops
+    dt, S, H, Hkv = DT_BFLOAT16, 512, 8, 2
+    q, k, v = (to_dev(normal_bits(s, (S, h, 128), dt)) for s, h in ((21, H), (22, Hkv), (23, Hkv)))
+    o_a, o_b = dev_empty((S, H, 128)), dev_empty((S, H, 128))
+    probe = torch.zeros(2, dtype=torch.int64, device="cuda")
+    ops.hip_flash_attn_gqa_layer(o_a, q, k, v, S, S, 0, H // Hkv, Hkv, 128, dt)
+    ops.hip_flash_attn_gqa_clocked_layer(o_b, q, k, v, S, S, 0, H // Hkv, Hkv, 128, dt, probe)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(o_a), to_host(o_b))
+    ticks, ref = (int(x) for x in probe.cpu())
+    assert ticks > 0 and ref > 0 and 300.0 < ticks / ref * 100.0 < 3000.0   # MHz
+    # decode-sized shapes are refused by the clocked entry (it times the prefill kernel only)
+    assert ops.lib.llmhip_flash_attn_gqa_clocked(o_b.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), 1, S,
+                                                 S - 1, H // Hkv, Hkv, 128, dt, probe.data_ptr(), None) == -2
+    alone, mix = ops.probe_mfma_ceiling(0, 5.0), ops.probe_mfma_ceiling(1, 5.0)
+    assert 250.0 < mix < alone < 2600.0, (alone, mix)
+    cus, mhz, mem = ops.device_props(0)
+    assert cus >= 64 and 1000.0 <= mhz <= 3000.0 and mem > (16 << 30)

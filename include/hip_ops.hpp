@@ -117,4 +117,28 @@ inline void hip_rope_kv_append_layer(void *output_q_dev, void *k_cache_dev, void
                                      stream));
 }
 
+// Batched decode: one query token for each of `batch` sequences that each own a cache of
+// kv_seq_stride rows (n valid).  No counterpart in the reference header, where decode is
+// npu_flash_attn_gqa_layer with m = 1 (src/llama2_layer_npu.cpp:866-869) and batch is always 1.
+// workspace_dev: llmhip_flash_decode_workspace_bytes(...) bytes of device memory owned by the caller.
+inline void hip_flash_decode_gqa_layer(void *output_dev, void *q_dev, void *k_cache_dev, void *v_cache_dev,
+                                       void *workspace_dev, size_t workspace_bytes, int batch, int n,
+                                       int64_t kv_seq_stride, int group_size, int kv_head_num, int head_dim,
+                                       int num_splits, DataType dt, gpuStream_t &stream) {
+  CHECK_LLMHIP(llmhip_flash_decode_gqa(output_dev, q_dev, k_cache_dev, v_cache_dev, workspace_dev,
+                                       workspace_bytes, batch, n, kv_seq_stride, group_size, kv_head_num,
+                                       head_dim, num_splits, dt, stream));
+}
+
+// The same decode for callers that cannot allocate or carry a workspace (HIP graph capture, serving
+// loops): the partials live in a fixed 4 MiB device array inside the library.
+inline void hip_flash_decode_gqa_static_layer(void *output_dev, void *q_dev, void *k_cache_dev,
+                                              void *v_cache_dev, int batch, int n, int64_t kv_seq_stride,
+                                              int group_size, int kv_head_num, int head_dim, int num_splits,
+                                              DataType dt, gpuStream_t &stream) {
+  CHECK_LLMHIP(llmhip_flash_decode_gqa_static(output_dev, q_dev, k_cache_dev, v_cache_dev, batch, n,
+                                              kv_seq_stride, group_size, kv_head_num, head_dim, num_splits,
+                                              dt, stream));
+}
+
 }  // namespace llm_simple_amd

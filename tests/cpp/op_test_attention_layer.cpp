@@ -1,7 +1,8 @@
 // Drives AttentionGPUImpl the way a model step drives a transformer layer's attention
 // block (src/llama2_layer_npu.cpp:780-869): one prefill of --prompt tokens, then
-// --steps decode steps with the KV cache growing in place, checked after every step
-// against the oracle's unfused rope -> append -> attention sequence.
+// --steps decode steps with the KV cache growing in place, then (--chunk N) one more chunk of N
+// tokens over the whole cache (chunked prefill), checked after every step against the oracle's
+// unfused rope -> append -> attention sequence.
 #include "op_test_common.hpp"
 
 using namespace llm_simple_amd;
@@ -10,6 +11,7 @@ int main(int argc, char **argv) {
   const int H = optest::flag_int(argc, argv, "head_num", 12), Hkv = optest::flag_int(argc, argv, "kv_head_num", 2);
   const int prompt = optest::flag_int(argc, argv, "prompt", 64), steps = optest::flag_int(argc, argv, "steps", 8);
   const int max_seq_len = optest::flag_int(argc, argv, "max_seq_len", 512);
+  const int chunk = optest::flag_int(argc, argv, "chunk", 0);
   const bool is_neox = optest::flag_int(argc, argv, "is_neox", 1) != 0;
   const float theta = std::atof(optest::flag(argc, argv, "theta", "1000000").c_str());
   const DataType dt = optest::parse_dtype(optest::flag(argc, argv, "dtype", "bf16"));
@@ -33,8 +35,9 @@ int main(int argc, char **argv) {
   const float tol = dt == DT_BFLOAT16 ? 1e-2f : 2e-3f;
   float worst = 0;
   size_t prev = 0;
-  for (int step = 0; step <= steps; ++step) {
-    const size_t cur = step == 0 ? prompt : prev + 1;
+  const int total_steps = steps + (chunk > 0 ? 1 : 0);
+  for (int step = 0; step <= total_steps; ++step) {
+    const size_t cur = step == 0 ? prompt : (step > steps ? prev + chunk : prev + 1);
     InferenceCtx ctx(cur, prev, stream);
     const size_t m = ctx.cur_size;
     auto q = optest::normal_bits(100 + step, m * H * hd, dt), k = optest::normal_bits(200 + step, m * Hkv * hd, dt),
@@ -66,7 +69,7 @@ int main(int argc, char **argv) {
   const size_t valid = prev * Hkv * hd;
   const bool caches_equal = std::memcmp(hk->data_ptr, kc.data(), valid * 2) == 0 &&
                             std::memcmp(hv->data_ptr, vc.data(), valid * 2) == 0;
-  std::printf("worst max-abs over %d steps: %.3e (bound %.0e); caches %s\n", steps + 1, worst, tol,
+  std::printf("worst max-abs over %d steps: %.3e (bound %.0e); caches %s\n", total_steps + 1, worst, tol,
               caches_equal ? "bit-identical" : "DIFFER");
   CHECK_LLMHIP(llmhip_stream_destroy(stream));
   const bool ok = worst <= tol && caches_equal && hip_last_status() == 0;

@@ -43,6 +43,9 @@ def test_op_test_rope_single(flags):
     ("--head_num", 12, "--kv_head_num", 2, "--prompt", 256, "--steps", 24, "--dtype", "bf16", "--is_neox", 1),  # config 3
     ("--head_num", 32, "--kv_head_num", 32, "--prompt", 40, "--steps", 6, "--dtype", "fp16", "--is_neox", 0,
      "--theta", 10000),
+    # chunked prefill through the layer: 64 more tokens over a 2403-row cache (key-range split, packed rows)
+    ("--head_num", 28, "--kv_head_num", 4, "--prompt", 2400, "--steps", 3, "--chunk", 64, "--max_seq_len", 2560,
+     "--dtype", "bf16", "--is_neox", 1),
 ])
 def test_attention_layer_prefill_then_decode(flags):
     _run("op_test_attention_layer", *flags)

@@ -29,10 +29,15 @@ extern "C" {
 #define LLMHIP_DT_BFLOAT16 5 /* prebuild/defs.hpp:14 */
 
 #define LLMHIP_OK 0
-#define LLMHIP_ERR_INVALID_ARG (-1)   /* null pointer, non-positive size, bad dtype */
+#define LLMHIP_ERR_INVALID_ARG (-1)   /* null or misaligned pointer, non-positive size, bad dtype */
 #define LLMHIP_ERR_UNSUPPORTED (-2)   /* head_dim != 128, group too large for the kernel */
 #define LLMHIP_ERR_WORKSPACE (-3)     /* workspace missing or too small */
 #define LLMHIP_ERR_NO_DEVICE (-4)     /* no HIP device visible */
+
+/* Every device pointer handed to the operators below must be 16-byte aligned (anything the
+ * runtime's allocator returns is; so is any row of a cache whose base is): the kernels move
+ * 16-byte pieces, and a misaligned pointer is rejected with LLMHIP_ERR_INVALID_ARG before any
+ * launch rather than left to fault on the device. */
 
 /* ------------------------------------------------------------------ */
 /* attention                                                           */

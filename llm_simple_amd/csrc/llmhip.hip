@@ -20,6 +20,9 @@ constexpr int kMaxDecodeSplits = 256;
 inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 inline int from_hip(hipError_t e) { return e == hipSuccess ? LLMHIP_OK : (int)e; }
 inline bool dtype_ok(int dt) { return dt == LLMHIP_DT_FLOAT16 || dt == LLMHIP_DT_BFLOAT16; }
+// every kernel moves 16-byte pieces: a misaligned base pointer would fault on the device
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+template <typename... P> inline bool all_aligned16(P... ptrs) { return (aligned16(ptrs) && ...); }
 
 // Split-KV scratch for the entry points that mirror the reference signatures
 // and therefore have no workspace argument: one grow-only buffer per stream.
@@ -55,7 +58,7 @@ int scratch_for_locked(void *stream, size_t need, void **out) {
 int attn_common(void *out, const void *q, const void *k, const void *v, int m, int n,
                 int offset, int group_size, int kv_head_num, int head_dim, int dt,
                 void *stream) {
-  if (!out || !q || !k || !v) return LLMHIP_ERR_INVALID_ARG;
+  if (!out || !q || !k || !v || !all_aligned16(out, q, k, v)) return LLMHIP_ERR_INVALID_ARG;
   if (m < 1 || n < 1 || offset < 0 || group_size < 1 || kv_head_num < 1)
     return LLMHIP_ERR_INVALID_ARG;
   if (!dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
@@ -116,7 +119,9 @@ int llmhip_flash_attn_opt_prefill(void *out, const void *q, const void *k, const
 int llmhip_flash_attn_gqa_clocked(void *out, const void *q, const void *k, const void *v, int m,
                                   int n, int offset, int group_size, int kv_head_num, int head_dim,
                                   int dt, void *clock_probe, void *stream) {
-  if (!out || !q || !k || !v || !clock_probe) return LLMHIP_ERR_INVALID_ARG;
+  if (!out || !q || !k || !v || !clock_probe || !all_aligned16(out, q, k, v) ||
+      (reinterpret_cast<uintptr_t>(clock_probe) & 7u))
+    return LLMHIP_ERR_INVALID_ARG;
   if (m < 1 || n < 1 || offset < 0 || group_size < 1 || kv_head_num < 1 || !dtype_ok(dt))
     return LLMHIP_ERR_INVALID_ARG;
   if (head_dim != 128) return LLMHIP_ERR_UNSUPPORTED;
@@ -158,7 +163,8 @@ int llmhip_flash_decode_gqa(void *out, const void *q, const void *k_cache,
                             int batch, int n, int64_t kv_seq_stride, int group_size,
                             int kv_head_num, int head_dim, int num_splits, int dt,
                             void *stream) {
-  if (!out || !q || !k_cache || !v_cache) return LLMHIP_ERR_INVALID_ARG;
+  if (!out || !q || !k_cache || !v_cache || !all_aligned16(out, q, k_cache, v_cache, workspace))
+    return LLMHIP_ERR_INVALID_ARG;
   if (batch < 1 || n < 1 || group_size < 1 || kv_head_num < 1 || kv_seq_stride < n)
     return LLMHIP_ERR_INVALID_ARG;
   if (!dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
@@ -176,7 +182,8 @@ int llmhip_flash_decode_gqa(void *out, const void *q, const void *k_cache,
 int llmhip_flash_decode_gqa_static(void *out, const void *q, const void *k_cache, const void *v_cache,
                                    int batch, int n, int64_t kv_seq_stride, int group_size,
                                    int kv_head_num, int head_dim, int num_splits, int dt, void *stream) {
-  if (!out || !q || !k_cache || !v_cache) return LLMHIP_ERR_INVALID_ARG;
+  if (!out || !q || !k_cache || !v_cache || !all_aligned16(out, q, k_cache, v_cache))
+    return LLMHIP_ERR_INVALID_ARG;
   if (batch < 1 || n < 1 || group_size < 1 || kv_head_num < 1 || kv_seq_stride < n)
     return LLMHIP_ERR_INVALID_ARG;
   if (!dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
@@ -196,7 +203,8 @@ size_t llmhip_flash_decode_static_scratch_bytes(void) { return kStaticDecodeScra
 int llmhip_rope(void *out_q, void *out_k, const void *freq_cis, const void *in_q,
                 const void *in_k, int start_pos, int cur_size, int n_heads, int hidden_dim,
                 int is_neox_style, int dt, void *stream) {
-  if (!out_q || !out_k || !freq_cis || !in_q || !in_k) return LLMHIP_ERR_INVALID_ARG;
+  if (!out_q || !out_k || !freq_cis || !in_q || !in_k || !all_aligned16(out_q, out_k, freq_cis, in_q, in_k))
+    return LLMHIP_ERR_INVALID_ARG;
   if (start_pos < 0 || cur_size < 1 || n_heads < 1 || !dtype_ok(dt))
     return LLMHIP_ERR_INVALID_ARG;
   if (hidden_dim != n_heads * 128) return LLMHIP_ERR_UNSUPPORTED;
@@ -208,7 +216,7 @@ int llmhip_rope(void *out_q, void *out_k, const void *freq_cis, const void *in_q
 int llmhip_rope_single(void *out, const void *freq_cis, const void *in, int start_pos,
                        int cur_size, int n_heads, int hidden_dim, int is_neox_style, int dt,
                        void *stream) {
-  if (!out || !freq_cis || !in) return LLMHIP_ERR_INVALID_ARG;
+  if (!out || !freq_cis || !in || !all_aligned16(out, freq_cis, in)) return LLMHIP_ERR_INVALID_ARG;
   if (start_pos < 0 || cur_size < 1 || n_heads < 1 || !dtype_ok(dt))
     return LLMHIP_ERR_INVALID_ARG;
   if (hidden_dim != n_heads * 128) return LLMHIP_ERR_UNSUPPORTED;
@@ -221,7 +229,8 @@ int llmhip_rope_kv_append(void *out_q, void *k_cache, void *v_cache, const void 
                           const void *in_q, const void *in_k, const void *in_v,
                           int start_pos, int cur_size, int n_heads, int n_kv_heads,
                           int head_dim, int is_neox_style, int dt, void *stream) {
-  if (!out_q || !k_cache || !v_cache || !freq_cis || !in_q || !in_k || !in_v)
+  if (!out_q || !k_cache || !v_cache || !freq_cis || !in_q || !in_k || !in_v ||
+      !all_aligned16(out_q, k_cache, v_cache, freq_cis, in_q, in_k, in_v))
     return LLMHIP_ERR_INVALID_ARG;
   if (start_pos < 0 || cur_size < 1 || n_heads < 1 || n_kv_heads < 1 || !dtype_ok(dt))
     return LLMHIP_ERR_INVALID_ARG;
@@ -380,7 +389,8 @@ int llmhip_matmul_bias(void *out, const void *lhs, const void *weight, const voi
 }
 int llmhip_add(void *out, const void *lhs, const void *rhs, long long total_size, int dt,
                void *stream) {
-  if (!out || !lhs || !rhs || total_size < 0 || !dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
+  if (!out || !lhs || !rhs || total_size < 0 || !dtype_ok(dt) || !all_aligned16(out, lhs, rhs))
+    return LLMHIP_ERR_INVALID_ARG;
   return from_hip(launch_add(out, lhs, rhs, (size_t)total_size, dt, as_stream(stream)));
 }
 

@@ -122,10 +122,11 @@ static void test_freq_cis() {
 }
 
 static void test_abi_validation() {
-  char x[16];
-  void *p = x;
+  alignas(16) char x[32];
+  void *p = x;  // 16-byte aligned: misaligned pointers are refused as invalid arguments
   // rejected before any launch, with or without a device
   EXPECT(llmhip_flash_attn(nullptr, p, p, p, 1, 1, 0, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
+  EXPECT(llmhip_flash_attn(p, x + 2, p, p, 1, 1, 0, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);  // misaligned q
   EXPECT(llmhip_flash_attn(p, p, p, p, 0, 1, 0, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
   EXPECT(llmhip_flash_attn(p, p, p, p, 1, 0, 0, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);
   EXPECT(llmhip_flash_attn(p, p, p, p, 1, 1, -1, 1, 128, 4, nullptr) == LLMHIP_ERR_INVALID_ARG);

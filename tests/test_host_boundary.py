@@ -36,14 +36,21 @@ def test_cpp_overloads_cover_reference_operator_names():
 
 def test_argument_validation_without_gpu():
     import llm_simple_amd.ops as ops
-    buf = ctypes.create_string_buffer(64)
-    p = ctypes.addressof(buf)
+    buf = ctypes.create_string_buffer(96)
+    p = (ctypes.addressof(buf) + 15) & ~15
     lib = ops.lib
     assert lib.llmhip_flash_attn(None, p, p, p, 1, 1, 0, 1, 128, 4, None) == -1
     assert lib.llmhip_flash_attn(p, p, p, p, 1, 1, 0, 1, 64, 4, None) == -2
     assert lib.llmhip_flash_attn_gqa(p, p, p, p, 1, 1, 0, 1, 1, 128, 7, None) == -1
     assert lib.llmhip_flash_decode_gqa(p, p, p, p, None, 0, 1, 4096, 4096, 5, 8, 128, 4, 5, None) == -3
     assert lib.llmhip_rope_single(p, p, p, 0, 1, 2, 100, 0, 4, None) == -2
+    # misaligned device pointers are refused before any launch (the kernels move 16-byte pieces)
+    assert p % 16 == 0
+    assert lib.llmhip_flash_attn(p, p + 2, p, p, 1, 1, 0, 1, 128, 4, None) == -1
+    assert lib.llmhip_flash_attn_gqa(p + 8, p, p, p, 1, 1, 0, 1, 1, 128, 4, None) == -1
+    assert lib.llmhip_rope_single(p, p + 4, p, 0, 1, 2, 256, 0, 4, None) == -1
+    assert lib.llmhip_rope_kv_append(p, p, p + 6, p, p, p, p, 0, 1, 1, 1, 128, 0, 4, None) == -1
+    assert lib.llmhip_flash_decode_gqa_static(p, p, p + 2, p, 1, 16, 16, 5, 8, 128, 1, 5, None) == -1
     try:
         ops.hip_flash_attn_layer(0, p, p, p, 1, 1, 0, 1, 128, 4)
     except ops.LlmHipError as e:

@@ -62,8 +62,8 @@ def test_static_decode_rejects_what_does_not_fit():
     lib = ops.lib
     cap = lib.llmhip_flash_decode_static_scratch_bytes()
     assert cap == 4 << 20
-    buf = ctypes.create_string_buffer(64)
-    p = ctypes.addressof(buf)
+    buf = ctypes.create_string_buffer(96)
+    p = (ctypes.addressof(buf) + 15) & ~15  # the entry points refuse misaligned pointers
     # 64 sequences x 8 kv heads x 2 splits = 1024 slots of 8320 bytes > 4 MiB: rejected before any launch
     assert ops.flash_decode_workspace_bytes(64, 5, 8, 128, 2) > cap
     assert lib.llmhip_flash_decode_gqa_static(p, p, p, p, 64, 4096, 4096, 5, 8, 128, 2, DT_BFLOAT16, None) == -3

@@ -235,6 +235,41 @@ def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
             "gbs_hot": kv_bytes / (hot_ms * 1e-3) / 1e9, "max_abs_err": worst}
 
 
+def bench_decode_step(ops, torch, timer, n, steps, warmup, H=40, Hkv=8):
+    """What one layer does per generated token (src/llama2_layer_npu.cpp:780-869, batch 1): the new token's
+    q and k rotated, k and v appended at row n-1, attention of the one query row over the n cache rows --
+    the fused rope + append launch and the reference-signature attention call (split-KV decode + combine),
+    and the same step with rope and append inside the decode kernel (llmhip_decode_step_gqa)."""
+    import numpy as np
+    g = torch.Generator(device="cuda").manual_seed(1005 + n)
+    bf = torch.bfloat16
+    nbuf = max(2, -(-(1 << 30) // (2 * n * Hkv * 256)) + 1)
+    kcs = [torch.randn(n, Hkv, 128, device="cuda", dtype=bf, generator=g) for _ in range(nbuf)]
+    vcs = [torch.randn(n, Hkv, 128, device="cuda", dtype=bf, generator=g) for _ in range(nbuf)]
+    q = torch.randn(1, H, 128, device="cuda", dtype=bf, generator=g)
+    k = torch.randn(1, Hkv, 128, device="cuda", dtype=bf, generator=g)
+    v = torch.randn(1, Hkv, 128, device="cuda", dtype=bf, generator=g)
+    qe, out = torch.empty_like(q), torch.empty_like(q)
+    table = torch.from_numpy(np.ascontiguousarray(ops.init_freq_cis(128, n, 1e6, DT_BF16))).cuda()
+
+    def step(i):
+        j = i % nbuf
+        ops.hip_rope_kv_append_layer(qe, kcs[j], vcs[j], table, q, k, v, n - 1, 1, H, Hkv, 128, True, DT_BF16)
+        ops.hip_flash_attn_gqa_layer(out, qe, kcs[j], vcs[j], 1, n, n - 1, H // Hkv, Hkv, 128, DT_BF16)
+
+    def fused(i):
+        j = i % nbuf
+        ops.hip_decode_step_gqa_layer(out, kcs[j], vcs[j], table, q, k, v, n - 1, H // Hkv, Hkv, 128, True, DT_BF16)
+
+    settle(torch, step, warmup)
+    ms, _, _ = timed(torch, timer, step, max(steps, MIN_REPS))
+    want = host_bits(out).copy()
+    ms_f, _, _ = timed(torch, timer, fused, max(steps, MIN_REPS))
+    same = bool((host_bits(out) == want).all())  # both paths left the result of the same buffer in `out`
+    return {"n": n, "H": H, "Hkv": Hkv, "us_three_launches": ms * 1e3, "us_fused": ms_f * 1e3,
+            "fused_output_bit_identical": same, "kv_gbs_fused": 2.0 * n * Hkv * 256 / (ms_f * 1e-3) / 1e9}
+
+
 def bench_rope_append(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
     import numpy as np
     g = torch.Generator(device="cuda").manual_seed(7)
@@ -436,6 +471,11 @@ def main():
             "traffic_source": TRAFFIC_SOURCE, "max_abs_err": head["max_abs_err"],
             "workload": f"Qwen2.5-32B decode bf16 H=40 Hkv=8 n={head['n']} batch={head['batch']} "
                         f"({head['kv_bytes'] / 2 ** 20:.0f} MiB of K+V per launch, cold)"}
+        extra["decode_step"] = [bench_decode_step(ops, torch, timer, n, args.steps, args.warmup) for n in (4096, 32768)]
+        for r in extra["decode_step"]:
+            log(f"decode step B=1 n={r['n']}: rope+append, decode, combine {r['us_three_launches']:.1f} us; fused into the "
+                f"decode kernel {r['us_fused']:.1f} us ({r['kv_gbs_fused']:.0f} GB/s), bit-identical {r['fused_output_bit_identical']}")
+        torch.cuda.empty_cache()
         extra["decode_all"] = [
             {"batch": r["batch"], "n": r["n"], "splits": r["splits"], "us_cold": r["ms_cold"] * 1e3,
              "gbs_cold": r["gbs_cold"], "frac_cold": r["gbs_cold"] / PEAK_HBM_GBS,

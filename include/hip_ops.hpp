@@ -141,4 +141,15 @@ inline void hip_flash_decode_gqa_static_layer(void *output_dev, void *q_dev, voi
                                               dt, stream));
 }
 
+// One decode step in one pass over the cache: the two npu_rope_single_layer calls, the two cache
+// copies and npu_flash_attn_gqa_layer(m = 1) of src/llama2_layer_npu.cpp:790-869 in one operator.
+inline void hip_decode_step_gqa_layer(void *output_dev, void *k_cache_dev, void *v_cache_dev,
+                                      void *freqs_cis_dev, void *input_q_dev, void *input_k_dev,
+                                      void *input_v_dev, int pos, int group_size, int kv_head_num, int head_dim,
+                                      bool is_neox_style, DataType dt, gpuStream_t &stream) {
+  CHECK_LLMHIP(llmhip_decode_step_gqa(output_dev, k_cache_dev, v_cache_dev, freqs_cis_dev, input_q_dev,
+                                      input_k_dev, input_v_dev, pos, group_size, kv_head_num, head_dim,
+                                      is_neox_style ? 1 : 0, dt, stream));
+}
+
 }  // namespace llm_simple_amd

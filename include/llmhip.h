@@ -131,6 +131,21 @@ int llmhip_flash_decode_gqa_static(void *out, const void *q, const void *k_cache
                                    int dt, void *stream);
 size_t llmhip_flash_decode_static_scratch_bytes(void);
 
+/* One decode step of one sequence in a single pass over the cache: what the reference does per
+ * generated token with four calls -- npu_rope_single_layer on q and on k, two cache copies and
+ * npu_flash_attn_gqa_layer with m = 1 (src/llama2_layer_npu.cpp:790-798, :830-844, :866-869) --
+ * with the rotary embedding and the append inside the decode kernel.  in_q [group_size*kv_head_num]
+ * [head_dim], in_k, in_v [kv_head_num][head_dim]: the projections of the token at position pos,
+ * unrotated.  Rows [0, pos) of the caches are read; row pos of k_cache receives rope(in_k), row pos
+ * of v_cache receives in_v; out = attention of rope(in_q) over rows [0, pos].  The results (output
+ * and both cache rows) are bit-identical to llmhip_rope_kv_append(start_pos = pos, cur_size = 1)
+ * followed by llmhip_flash_attn_gqa(m = 1, n = pos + 1, offset = pos).  Split-KV partials come from
+ * the same per-stream scratch as llmhip_flash_attn_gqa. */
+int llmhip_decode_step_gqa(void *out, void *k_cache, void *v_cache, const void *freq_cis,
+                           const void *in_q, const void *in_k, const void *in_v, int pos,
+                           int group_size, int kv_head_num, int head_dim, int is_neox_style, int dt,
+                           void *stream);
+
 /* ------------------------------------------------------------------ */
 /* rotary embedding and KV-cache append                                */
 /* ------------------------------------------------------------------ */

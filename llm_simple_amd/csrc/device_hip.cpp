@@ -186,13 +186,20 @@ std::shared_ptr<Tensor> AttentionGPUImpl::Forward(std::shared_ptr<Tensor> q,
   auto out = Tensor::MakeGPUTensor(static_cast<size_t>(hidden) * cur_size, dtype_);
   if (!q_emb || !out || !q_emb->data_ptr || !out->data_ptr) return nullptr;  // nothing launched yet
   hip_last_status() = 0;
-  hip_rope_kv_append_layer(q_emb->data_ptr, k_cache->data_ptr, v_cache->data_ptr,
-                           freq_cis_->data_ptr, q->data_ptr, k->data_ptr, v->data_ptr,
-                           static_cast<int>(ctx.prev_pos), cur_size, n_heads_, n_kv_heads_,
-                           head_dim_, neox_, dtype_, ctx.gpu_stream);
-  hip_flash_attn_gqa_layer(out->data_ptr, q_emb->data_ptr, k_cache->data_ptr, v_cache->data_ptr,
-                           cur_size, static_cast<int>(ctx.cur_pos), static_cast<int>(ctx.prev_pos),
-                           n_heads_ / n_kv_heads_, n_kv_heads_, head_dim_, dtype_, ctx.gpu_stream);
+  if (cur_size == 1 && n_heads_ / n_kv_heads_ <= 16) {
+    // a decode step: rotary embedding, append and attention in one pass over the cache
+    hip_decode_step_gqa_layer(out->data_ptr, k_cache->data_ptr, v_cache->data_ptr, freq_cis_->data_ptr,
+                              q->data_ptr, k->data_ptr, v->data_ptr, static_cast<int>(ctx.prev_pos),
+                              n_heads_ / n_kv_heads_, n_kv_heads_, head_dim_, neox_, dtype_, ctx.gpu_stream);
+  } else {
+    hip_rope_kv_append_layer(q_emb->data_ptr, k_cache->data_ptr, v_cache->data_ptr,
+                             freq_cis_->data_ptr, q->data_ptr, k->data_ptr, v->data_ptr,
+                             static_cast<int>(ctx.prev_pos), cur_size, n_heads_, n_kv_heads_,
+                             head_dim_, neox_, dtype_, ctx.gpu_stream);
+    hip_flash_attn_gqa_layer(out->data_ptr, q_emb->data_ptr, k_cache->data_ptr, v_cache->data_ptr,
+                             cur_size, static_cast<int>(ctx.cur_pos), static_cast<int>(ctx.prev_pos),
+                             n_heads_ / n_kv_heads_, n_kv_heads_, head_dim_, dtype_, ctx.gpu_stream);
+  }
   // q_emb goes back to the pool when this scope ends while the attention launch may
   // still read it: drain the stream first, the rule the reference states at
   // src/llama2_layer_npu.cpp:605-608.

@@ -53,7 +53,57 @@ struct DecodeParams {
   int rows;  // m * g
   int num_splits, chunk;
   float scale_log2e;
+  // Fused decode step (FUSED kernels only): the token at row fused_pos = n - 1 is not in the cache yet.
+  // q, new_k and new_v hold the unrotated projections of that token ([H][128], [Hkv][128] twice);
+  // q and the new K row are rotated with table row freq_row (64 (cos, sin) pairs) as they are loaded,
+  // and the workgroup that owns the last key range writes the rotated K row and the V row to the cache.
+  const char *new_k;
+  const char *new_v;
+  const float *freq_row;
+  int fused_pos, is_neox;
 };
+
+// RoPE of the four 16-byte fragments a lane holds of one head row: fragment kk = dims 8*cg + 32*kk .. +7.
+// Arithmetic of the rotary kernel, unfused products and sums (src/llama2_layer_cpu.cpp:835-856):
+// (a*c - b*s, a*s + b*c) rounded once; interleaved pairs (2f, 2f+1), neox pairs (f, f+64).
+template <typename T>
+__device__ __forceinline__ void rotate_frags(u32x4_t (&f)[4], const float *tab, int cg, int is_neox) {
+#pragma clang fp contract(off)
+  using E = Elem<T>;
+  auto get = [](const u32x4_t &w, int e) { return (uint16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu); };
+  auto put = [](u32x4_t &w, int e, uint16_t v) {
+    w[e >> 1] = (w[e >> 1] & ~(0xFFFFu << ((e & 1) * 16))) | ((uint32_t)v << ((e & 1) * 16));
+  };
+  if (is_neox) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const int d0 = 8 * cg + 32 * kk;  // pair index of element 0: d0 < 64
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float a = E::widen(get(f[kk], e)), b = E::widen(get(f[kk + 2], e));
+        const float c = tab[2 * (d0 + e)], sn = tab[2 * (d0 + e) + 1];
+        const float ra = a * c - b * sn;
+        const float rb = a * sn + b * c;
+        put(f[kk], e, E::round(ra));
+        put(f[kk + 2], e, E::round(rb));
+      }
+    }
+  } else {
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int f0 = (8 * cg + 32 * kk) / 2;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float a = E::widen(get(f[kk], 2 * j)), b = E::widen(get(f[kk], 2 * j + 1));
+        const float c = tab[2 * (f0 + j)], sn = tab[2 * (f0 + j) + 1];
+        const float ra = a * c - b * sn;
+        const float rb = a * sn + b * c;
+        put(f[kk], 2 * j, E::round(ra));
+        put(f[kk], 2 * j + 1, E::round(rb));
+      }
+    }
+  }
+}
 
 // V staging swizzle for the 16x16x32 transposed reads: one instruction touches
 // 8 rows x 32 bytes per half-wave, so the 32-byte slot index is XORed with
@@ -62,7 +112,7 @@ __device__ __forceinline__ int v_swizzle32_off(int row, int granule) {
   return row * kRowBytes + ((((granule >> 1) ^ (row & 7)) << 5) | ((granule & 1) << 4));
 }
 
-template <typename T>
+template <typename T, bool FUSED>
 __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams p) {
   using E = Elem<T>;
   __shared__ __attribute__((aligned(16))) char lds[4 * kDecWaveLds + 4 * kDecCols * 2 * 4];
@@ -95,6 +145,7 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
       u32x4_t z = {0u, 0u, 0u, 0u};
       qf[kk] = col_valid ? global_load_b128(qp + kk * 64) : z;
     }
+    if (FUSED && col_valid) rotate_frags<T>(qf, p.freq_row, cg, p.is_neox);
   }
 
   f32x4_t o[8];
@@ -111,13 +162,16 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
     for (int blk = 0; blk < 2; ++blk) {
       const int key = min(kb0 + blk * 16 + col, p.n - 1);
       const char *kp = kbase + (size_t)key * kv_row_bytes + cg * 16;
+      if (FUSED && key == p.fused_pos) kp = p.new_k + (size_t)kvh * kRowBytes + cg * 16;
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) kn[blk][kk] = global_load_b128(kp + kk * 64);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int key = min(kb0 + 4 * i + cg, p.n - 1);
-      vn[i] = global_load_b128(vbase + (size_t)key * kv_row_bytes + col * 16);
+      const char *vp = vbase + (size_t)key * kv_row_bytes + col * 16;
+      if (FUSED && key == p.fused_pos) vp = p.new_v + (size_t)kvh * kRowBytes + col * 16;
+      vn[i] = global_load_b128(vp);
     }
   };
 
@@ -134,10 +188,32 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int i = 0; i < 8; ++i) lds_write_b128(vl, v_swizzle32_off(4 * i + cg, col), vn[i]);
+    if (FUSED && kb0 < k_end) {  // the new token's V row goes to the cache (vn is refilled below)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int key = min(kb0 + 4 * i + cg, p.n - 1);
+        if (key == p.fused_pos)
+          *reinterpret_cast<u32x4_t *>(const_cast<char *>(vbase) + (size_t)key * kv_row_bytes + col * 16) = vn[i];
+      }
+    }
     __builtin_amdgcn_wave_barrier();
     if (it + 1 < iters) issue_loads(it + 1);
 
     if (kb0 < k_end) {
+      if (FUSED) {
+        // the new token's row: rotate K in registers and append both rows to the cache (lanes whose
+        // clamped key is the new row all hold and write the same bytes)
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+          const int key = min(kb0 + blk * 16 + col, p.n - 1);
+          if (key == p.fused_pos) {
+            rotate_frags<T>(kc[blk], p.freq_row, cg, p.is_neox);
+            char *dst = const_cast<char *>(kbase) + (size_t)key * kv_row_bytes + cg * 16;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) *reinterpret_cast<u32x4_t *>(dst + kk * 64) = kc[blk][kk];
+          }
+        }
+      }
       // ---- S^T = K Q^T : 2 blocks of 16 keys ----
       f32x4_t s[2];
 #pragma unroll
@@ -363,11 +439,41 @@ size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_hea
   return slots * (kHeadDim + 2) * sizeof(float);
 }
 
+static hipError_t launch_decode_impl(DecodeParams &p, void *workspace, int batch, int kv_head_num, int num_splits,
+                                     int dt, bool fused, hipStream_t stream) {
+  p.chunk = decode_chunk(p.n, num_splits);
+  p.num_splits = (p.n + p.chunk - 1) / p.chunk;  // never more than asked for
+  p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
+  const size_t slots = (size_t)batch * kv_head_num * p.num_splits * kDecCols;
+  p.ws_o = static_cast<float *>(workspace);
+  p.ws_ml = p.ws_o ? p.ws_o + slots * kHeadDim : nullptr;
+  dim3 grid(p.num_splits, kv_head_num, batch);
+  if (dt == kDtFloat16) {
+    if (fused)
+      hipLaunchKernelGGL((flash_decode_kernel<_Float16, true>), grid, dim3(kDecThreads), 0, stream, p);
+    else
+      hipLaunchKernelGGL((flash_decode_kernel<_Float16, false>), grid, dim3(kDecThreads), 0, stream, p);
+  } else {
+    if (fused)
+      hipLaunchKernelGGL((flash_decode_kernel<__bf16, true>), grid, dim3(kDecThreads), 0, stream, p);
+    else
+      hipLaunchKernelGGL((flash_decode_kernel<__bf16, false>), grid, dim3(kDecThreads), 0, stream, p);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || p.num_splits == 1) return e;
+  dim3 cgrid(p.rows, kv_head_num, batch);
+  if (dt == kDtFloat16)
+    hipLaunchKernelGGL(flash_decode_combine_kernel<_Float16>, cgrid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL(flash_decode_combine_kernel<__bf16>, cgrid, dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
 hipError_t launch_flash_decode(void *out, const void *q, const void *k, const void *v,
                                void *workspace, int batch, int m, int n, int offset,
                                int64_t kv_seq_stride, int group_size, int kv_head_num,
                                int num_splits, int dt, hipStream_t stream) {
-  DecodeParams p;
+  DecodeParams p = {};
   p.q = static_cast<const char *>(q);
   p.k = static_cast<const char *>(k);
   p.v = static_cast<const char *>(v);
@@ -381,25 +487,35 @@ hipError_t launch_flash_decode(void *out, const void *q, const void *k, const vo
   p.Hkv = kv_head_num;
   p.H = group_size * kv_head_num;
   p.rows = m * group_size;
-  p.chunk = decode_chunk(n, num_splits);
-  p.num_splits = (n + p.chunk - 1) / p.chunk;  // never more than asked for
-  p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
-  const size_t slots = (size_t)batch * kv_head_num * p.num_splits * kDecCols;
-  p.ws_o = static_cast<float *>(workspace);
-  p.ws_ml = p.ws_o ? p.ws_o + slots * kHeadDim : nullptr;
-  dim3 grid(p.num_splits, kv_head_num, batch);
-  if (dt == kDtFloat16)
-    hipLaunchKernelGGL(flash_decode_kernel<_Float16>, grid, dim3(kDecThreads), 0, stream, p);
-  else
-    hipLaunchKernelGGL(flash_decode_kernel<__bf16>, grid, dim3(kDecThreads), 0, stream, p);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess || p.num_splits == 1) return e;
-  dim3 cgrid(p.rows, kv_head_num, batch);
-  if (dt == kDtFloat16)
-    hipLaunchKernelGGL(flash_decode_combine_kernel<_Float16>, cgrid, dim3(256), 0, stream, p);
-  else
-    hipLaunchKernelGGL(flash_decode_combine_kernel<__bf16>, cgrid, dim3(256), 0, stream, p);
-  return hipGetLastError();
+  return launch_decode_impl(p, workspace, batch, kv_head_num, num_splits, dt, false, stream);
+}
+
+// One decode step of one sequence with the rotary embedding and the cache append inside the decode
+// kernel: rows [0, pos) of the caches are read, row pos is produced from in_k / in_v and written.
+hipError_t launch_flash_decode_step(void *out, void *k_cache, void *v_cache, const void *freq_cis,
+                                    const void *in_q, const void *in_k, const void *in_v, void *workspace,
+                                    int pos, int group_size, int kv_head_num, int is_neox, int num_splits,
+                                    int dt, hipStream_t stream) {
+  DecodeParams p = {};
+  p.q = static_cast<const char *>(in_q);
+  p.k = static_cast<const char *>(k_cache);
+  p.v = static_cast<const char *>(v_cache);
+  p.out = static_cast<char *>(out);
+  p.batch = 1;
+  p.m = 1;
+  p.n = pos + 1;
+  p.offset = pos;
+  p.kv_seq_stride = pos + 1;
+  p.g = group_size;
+  p.Hkv = kv_head_num;
+  p.H = group_size * kv_head_num;
+  p.rows = group_size;
+  p.new_k = static_cast<const char *>(in_k);
+  p.new_v = static_cast<const char *>(in_v);
+  p.freq_row = static_cast<const float *>(freq_cis) + (size_t)pos * kHeadDim;
+  p.fused_pos = pos;
+  p.is_neox = is_neox ? 1 : 0;
+  return launch_decode_impl(p, workspace, 1, kv_head_num, num_splits, dt, true, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -25,6 +25,14 @@ hipError_t launch_flash_decode(void *out, const void *q, const void *k, const vo
                                int64_t kv_seq_stride, int group_size, int kv_head_num,
                                int num_splits, int dt, hipStream_t stream);
 
+// One decode step of one sequence, rotary embedding and cache append fused into the decode kernel:
+// q and the new K row are rotated with row `pos` of the table as they are loaded, the workgroups that own
+// the last key range write row pos of both caches, attention runs over rows [0, pos].
+hipError_t launch_flash_decode_step(void *out, void *k_cache, void *v_cache, const void *freq_cis,
+                                    const void *in_q, const void *in_k, const void *in_v, void *workspace,
+                                    int pos, int group_size, int kv_head_num, int is_neox, int num_splits,
+                                    int dt, hipStream_t stream);
+
 // Same decode with the split-KV partials in a fixed device array of kStaticDecodeScratchBytes inside
 // the library: no allocation, no workspace argument.  The caller checks the size beforehand.
 constexpr size_t kStaticDecodeScratchBytes = 4u << 20;

@@ -200,6 +200,30 @@ int llmhip_flash_decode_gqa_static(void *out, const void *q, const void *k_cache
 
 size_t llmhip_flash_decode_static_scratch_bytes(void) { return kStaticDecodeScratchBytes; }
 
+int llmhip_decode_step_gqa(void *out, void *k_cache, void *v_cache, const void *freq_cis, const void *in_q,
+                           const void *in_k, const void *in_v, int pos, int group_size, int kv_head_num,
+                           int head_dim, int is_neox_style, int dt, void *stream) {
+  if (!out || !k_cache || !v_cache || !freq_cis || !in_q || !in_k || !in_v ||
+      !all_aligned16(out, k_cache, v_cache, freq_cis, in_q, in_k, in_v))
+    return LLMHIP_ERR_INVALID_ARG;
+  if (pos < 0 || pos == INT32_MAX || group_size < 1 || kv_head_num < 1 || !dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
+  if (head_dim != 128 || group_size > kMaxDecodeCols) return LLMHIP_ERR_UNSUPPORTED;
+  if (kv_head_num > 65535) return LLMHIP_ERR_UNSUPPORTED;
+  const int n = pos + 1;
+  const int splits = flash_decode_default_splits(1, n, kv_head_num);
+  const size_t need = flash_decode_workspace_bytes(1, 1, group_size, kv_head_num, splits);
+  if (!need)
+    return from_hip(launch_flash_decode_step(out, k_cache, v_cache, freq_cis, in_q, in_k, in_v, nullptr, pos,
+                                             group_size, kv_head_num, is_neox_style, splits, dt,
+                                             as_stream(stream)));
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  void *ws = nullptr;
+  int rc = scratch_for_locked(stream, need, &ws);
+  if (rc != LLMHIP_OK) return rc;
+  return from_hip(launch_flash_decode_step(out, k_cache, v_cache, freq_cis, in_q, in_k, in_v, ws, pos, group_size,
+                                           kv_head_num, is_neox_style, splits, dt, as_stream(stream)));
+}
+
 int llmhip_rope(void *out_q, void *out_k, const void *freq_cis, const void *in_q,
                 const void *in_k, int start_pos, int cur_size, int n_heads, int hidden_dim,
                 int is_neox_style, int dt, void *stream) {

@@ -30,6 +30,7 @@ SYMBOLS = {
     "llmhip_flash_decode_gqa": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i64, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_gqa_static": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i64, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_static_scratch_bytes": (_sz, []),
+    "llmhip_decode_step_gqa": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "llmhip_flash_decode_default_splits": (_i, [_i, _i, _i]),
     "llmhip_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
@@ -152,6 +153,17 @@ def hip_flash_decode_gqa_static_layer(output_dev, q_dev, k_cache_dev, v_cache_de
                                               _ptr(v_cache_dev), batch, n, kv_seq_stride, group_size,
                                               kv_head_num, head_dim, num_splits, dt, stream),
            "hip_flash_decode_gqa_static_layer")
+
+
+def hip_decode_step_gqa_layer(output_dev, k_cache_dev, v_cache_dev, freqs_cis_dev, input_q_dev, input_k_dev,
+                              input_v_dev, pos, group_size, kv_head_num, head_dim, is_neox_style, dt, stream=0):
+    """One decode step in one pass over the cache: rope(q), rope(k) -> k_cache[pos], v -> v_cache[pos] and
+    attention over rows [0, pos], fused into the decode kernel (src/llama2_layer_npu.cpp:790-869 does it
+    with four calls)."""
+    _check(lib.llmhip_decode_step_gqa(_ptr(output_dev), _ptr(k_cache_dev), _ptr(v_cache_dev),
+                                      _ptr(freqs_cis_dev), _ptr(input_q_dev), _ptr(input_k_dev),
+                                      _ptr(input_v_dev), pos, group_size, kv_head_num, head_dim,
+                                      int(bool(is_neox_style)), dt, stream), "hip_decode_step_gqa_layer")
 
 
 def flash_decode_workspace_bytes(batch, group_size, kv_head_num, head_dim, num_splits):

@@ -454,3 +454,41 @@ def test_flash_decode_random_shapes():
         ops.hip_flash_decode_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), ws, wsb, batch, n, stride, g, Hkv,
                                        128, 0, dt)
         check_attention(to_host(d_out), q, k, v, n, n - 1, dt, batch=True)
+
+
+@pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
+@pytest.mark.parametrize("is_neox", [False, True])
+@pytest.mark.parametrize("H,Hkv", [(12, 2), (32, 32), (40, 8), (28, 4)])
+def test_decode_step_fused_equals_unfused_chain(dt, is_neox, H, Hkv):
+    """llmhip_decode_step_gqa (rope + append inside the decode kernel) against the unfused sequence
+    rope_kv_append -> flash_attn_gqa(m=1): output, K-cache row and V-cache row bit-identical, at cache
+    lengths around every boundary of the kernel (one key, a 32-key wave step, a 128-key workgroup step, a
+    split boundary, many splits); untouched rows keep their bytes; and the output against the oracle."""
+    ops = _ops()
+    max_seq = 5000
+    theta = 1e6 if dt == DT_BFLOAT16 else 10000.0
+    table = orc.init_freq_cis(128, max_seq, theta, dt)
+    d_table = f32_dev(table)
+    kc0 = normal_bits(61, (max_seq, Hkv, 128), dt)
+    vc0 = normal_bits(62, (max_seq, Hkv, 128), dt)
+    for pos in (0, 1, 31, 32, 127, 128, 129, 1000, 4095, 4999):
+        q = normal_bits(7000 + pos, (1, H, 128), dt)
+        k = normal_bits(7100 + pos, (1, Hkv, 128), dt)
+        v = normal_bits(7200 + pos, (1, Hkv, 128), dt)
+        # unfused
+        kc_a, vc_a = to_dev(kc0), to_dev(vc0)
+        qe, o_a = dev_empty(q.shape), dev_empty(q.shape)
+        ops.hip_rope_kv_append_layer(qe, kc_a, vc_a, d_table, to_dev(q), to_dev(k), to_dev(v), pos, 1, H, Hkv, 128,
+                                     is_neox, dt)
+        ops.hip_flash_attn_gqa_layer(o_a, qe, kc_a, vc_a, 1, pos + 1, pos, H // Hkv, Hkv, 128, dt)
+        # fused
+        kc_b, vc_b = to_dev(kc0), to_dev(vc0)
+        o_b = dev_empty(q.shape)
+        ops.hip_decode_step_gqa_layer(o_b, kc_b, vc_b, d_table, to_dev(q), to_dev(k), to_dev(v), pos, H // Hkv, Hkv,
+                                      128, is_neox, dt)
+        assert np.array_equal(to_host(kc_b), to_host(kc_a)), f"K cache differs at pos {pos}"
+        assert np.array_equal(to_host(vc_b), to_host(vc_a)), f"V cache differs at pos {pos}"
+        assert np.array_equal(to_host(o_b), to_host(o_a)), f"output differs at pos {pos}"
+        if pos in (0, 129, 4999):
+            kc_h, vc_h = to_host(kc_b), to_host(vc_b)
+            check_attention(to_host(o_b), orc.rope(q, table, pos, is_neox, dt), kc_h, vc_h, pos + 1, pos, dt)

@@ -221,6 +221,11 @@ def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
     reps = max(steps, MIN_REPS)
     cold, _, _ = timed(torch, timer, step, reps)
     hot_ms, _, _ = timed(torch, timer, hot, reps)
+    # a kernel that only reads the same K and V arrays, cold like `step`: what the memory system delivers at
+    # this byte count (the better of its two launch shapes)
+    sink = torch.empty(ops.STREAM_READ_SINK_BYTES, dtype=torch.uint8, device="cuda")
+    read_ms = min(timed(torch, timer, lambda i, var=var: ops.probe_stream_read(ks[i % nbuf], vs[i % nbuf], sink, var),
+                        reps)[0] for var in (0, 1))
     torch.cuda.synchronize()
     # accuracy of the last timed (hot) launch: sequence 0 and the last one against the fp32 oracle
     import numpy as np
@@ -232,7 +237,8 @@ def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
         worst = max(worst, float(np.abs(orc.widen(ob[b], DT_BF16) - ref).max()))
     return {"batch": batch, "n": n, "splits": splits, "kv_bytes": kv_bytes, "buffers": nbuf,
             "ms_cold": cold, "ms_hot": hot_ms, "gbs_cold": kv_bytes / (cold * 1e-3) / 1e9,
-            "gbs_hot": kv_bytes / (hot_ms * 1e-3) / 1e9, "max_abs_err": worst}
+            "gbs_hot": kv_bytes / (hot_ms * 1e-3) / 1e9, "max_abs_err": worst,
+            "ms_plain_read": read_ms, "gbs_plain_read": kv_bytes / (read_ms * 1e-3) / 1e9}
 
 
 def bench_decode_step(ops, torch, timer, n, steps, warmup, H=40, Hkv=8):
@@ -458,7 +464,8 @@ def main():
             r = bench_decode(ops, torch, timer, batch, n, args.steps, args.warmup)
             log(f"decode B={batch} n={n} splits={r['splits']}: cold {r['ms_cold'] * 1e3:.1f} us "
                 f"{r['gbs_cold']:.0f} GB/s, hot {r['ms_hot'] * 1e3:.1f} us {r['gbs_hot']:.0f} GB/s, "
-                f"max-abs {r['max_abs_err']:.2e}")
+                f"max-abs {r['max_abs_err']:.2e}; a plain read of the same arrays, cold: "
+                f"{r['ms_plain_read'] * 1e3:.1f} us {r['gbs_plain_read']:.0f} GB/s")
             dec.append(r)
             torch.cuda.empty_cache()
         head = dec[0]
@@ -469,6 +476,10 @@ def main():
             "frac": head["gbs_cold"] / PEAK_HBM_GBS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(("decode", head["batch"], head["n"])),
             "traffic_source": TRAFFIC_SOURCE, "max_abs_err": head["max_abs_err"],
+            "box": {"plain_read_gbs": head["gbs_plain_read"],
+                    "frac_of_plain_read": head["gbs_cold"] / head["gbs_plain_read"],
+                    "plain_read": "a kernel that only reads the same K and V arrays once, cold, timed the same way "
+                                  "(llmhip_probe_stream_read)"},
             "workload": f"Qwen2.5-32B decode bf16 H=40 Hkv=8 n={head['n']} batch={head['batch']} "
                         f"({head['kv_bytes'] / 2 ** 20:.0f} MiB of K+V per launch, cold)"}
         extra["decode_step"] = [bench_decode_step(ops, torch, timer, n, args.steps, args.warmup) for n in (4096, 32768)]
@@ -479,7 +490,9 @@ def main():
         extra["decode_all"] = [
             {"batch": r["batch"], "n": r["n"], "splits": r["splits"], "us_cold": r["ms_cold"] * 1e3,
              "gbs_cold": r["gbs_cold"], "frac_cold": r["gbs_cold"] / PEAK_HBM_GBS,
-             "us_hot": r["ms_hot"] * 1e3, "gbs_hot": r["gbs_hot"], "max_abs_err": r["max_abs_err"]} for r in dec]
+             "us_hot": r["ms_hot"] * 1e3, "gbs_hot": r["gbs_hot"], "max_abs_err": r["max_abs_err"],
+             "us_plain_read": r["ms_plain_read"] * 1e3, "frac_of_plain_read": r["ms_plain_read"] / r["ms_cold"]}
+            for r in dec]
 
     if "rope" in legs:
         r = bench_rope_append(ops, torch, timer, args.seq, args.steps, args.warmup)

@@ -197,6 +197,15 @@ int llmhip_device_props(int device, int *compute_units, int *max_clock_khz, size
  * attention kernel with that instruction mix on this machine.  The benchmark prints both next to
  * the published peak.  Allocates and frees two small device buffers; runs on the default stream. */
 int llmhip_probe_mfma_ceiling(int mix, double target_ms, double *tflops);
+/* Measurement aid, no counterpart in the reference: a plain streaming read of two device arrays of
+ * bytes_each bytes (a multiple of 16), every byte read once and nothing else done -- what the memory
+ * system delivers to a kernel that only reads, to set beside the decode kernel's rate on the same byte
+ * count.  variant 0: one workgroup per CU with 8 loads in flight per thread; variant 1: two per CU with
+ * 4 (the better one below about 256 MiB).  sink: LLMHIP_STREAM_READ_SINK_BYTES bytes of device memory
+ * that receive a checksum per wave.  Asynchronous on `stream`; allocates nothing. */
+#define LLMHIP_STREAM_READ_SINK_BYTES 65536
+int llmhip_probe_stream_read(const void *src_a, const void *src_b, size_t bytes_each, void *sink,
+                             size_t sink_bytes, int variant, void *stream);
 int llmhip_set_device(int device);
 int llmhip_malloc(void **ptr, size_t bytes);
 int llmhip_free(void *ptr);

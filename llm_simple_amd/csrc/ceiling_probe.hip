@@ -76,6 +76,34 @@ __global__ __launch_bounds__(512, 1) void mfma_ceiling_kernel(const u32x4_t *ops
   out[(size_t)blockIdx.x * 512 + tid] = r;
 }
 
+// Plain streaming read of two arrays of n16 16-byte pieces each, every piece read once, U loads in flight
+// per thread, consecutive threads of the whole grid on consecutive pieces (all CUs walk through memory
+// together, which the DRAM channels serve best).  The XOR of everything read goes to sink[wave], so that
+// no load can be dropped.
+template <int U>
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t *__restrict__ a, const u32x4_t *__restrict__ b,
+                                                          size_t n16, unsigned *sink) {
+  const size_t total = (size_t)gridDim.x * 256;
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+#pragma unroll 1
+  for (int half = 0; half < 2; ++half) {
+    const u32x4_t *src = half ? b : a;
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    for (; i + (U - 1) * total < n16; i += U * total) {
+      u32x4_t v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = src[i + u * total];
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc ^= v[u];
+    }
+    for (; i < n16; i += total) acc ^= src[i];
+  }
+  unsigned r = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+#pragma unroll
+  for (int o = 32; o; o >>= 1) r ^= (unsigned)__shfl_xor((int)r, o, 64);
+  if ((threadIdx.x & 63) == 0) sink[blockIdx.x * 4 + (threadIdx.x >> 6)] = r;
+}
+
 // N(0,1) rounded to bf16 from a fixed counter-based generator (splitmix64 + Box-Muller).
 uint16_t normal_bf16(uint64_t i) {
   auto mix = [](uint64_t z) {
@@ -92,6 +120,30 @@ uint16_t normal_bf16(uint64_t i) {
 }
 
 }  // namespace
+
+// variant 0: one workgroup per CU, 8 loads in flight per thread (best from 256 MiB up); variant 1: two
+// per CU, 4 in flight (best below).  sink: 4 bytes per wave of the grid.
+hipError_t launch_stream_read(const void *a, const void *b, size_t bytes_each, void *sink, int variant,
+                              hipStream_t stream) {
+  static int cus_of[64] = {};  // per device; written once with the same value by whoever comes first
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+  int cus = cus_of[dev];
+  if (cus == 0) {
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess || cus <= 0) return e != hipSuccess ? e : hipErrorInvalidDevice;
+    cus_of[dev] = cus;
+  }
+  const u32x4_t *pa = static_cast<const u32x4_t *>(a), *pb = static_cast<const u32x4_t *>(b);
+  unsigned *ps = static_cast<unsigned *>(sink);
+  if (variant == 0)
+    hipLaunchKernelGGL(stream_read_kernel<8>, dim3(cus), dim3(256), 0, stream, pa, pb, bytes_each / 16, ps);
+  else
+    hipLaunchKernelGGL(stream_read_kernel<4>, dim3(2 * cus), dim3(256), 0, stream, pa, pb, bytes_each / 16, ps);
+  return hipGetLastError();
+}
 
 // Runs one of the two loops on every CU for about `target_ms` and returns the sustained TFLOP/s of
 // its MFMAs (0 on error).  Allocates and frees its own small buffers.

@@ -51,7 +51,7 @@ struct DecodeParams {
   int64_t kv_seq_stride;
   int g, Hkv, H;
   int rows;  // m * g
-  int num_splits, chunk;
+  int num_splits;
   float scale_log2e;
   // Fused decode step (FUSED kernels only): the token at row fused_pos = n - 1 is not in the cache yet.
   // q, new_k and new_v hold the unrotated projections of that token ([H][128], [Hkv][128] twice);
@@ -121,10 +121,13 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int col = lane & 15, cg = lane >> 4;
 
-  const int k_begin = split * p.chunk;
-  const int k_end = min(p.n, k_begin + p.chunk);
-  const int span = max(k_end - k_begin, 0);
-  const int iters = (span + kDecStepKeys - 1) / kDecStepKeys;
+  // A split is not a contiguous key range but every num_splits-th block of kDecStepKeys keys: the
+  // workgroups of one sequence then walk through its cache side by side, which the DRAM channels
+  // serve better than as many far-apart streams (the softmax merge does not care which keys a
+  // partial covers).
+  const int nblocks = (p.n + kDecStepKeys - 1) / kDecStepKeys;
+  const int k_end = p.n;
+  const int iters = (nblocks - split + p.num_splits - 1) / p.num_splits;  // blocks split, split + S, ...
 
   const size_t kv_row_bytes = (size_t)p.Hkv * kRowBytes;
   const size_t seq_off = (size_t)b * p.kv_seq_stride * kv_row_bytes + (size_t)kvh * kRowBytes;
@@ -157,7 +160,7 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
 
   u32x4_t kn[2][4], vn[8];
   auto issue_loads = [&](int it) {
-    const int kb0 = k_begin + it * kDecStepKeys + wave * kDecWaveKeys;
+    const int kb0 = (it * p.num_splits + split) * kDecStepKeys + wave * kDecWaveKeys;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
       const int key = min(kb0 + blk * 16 + col, p.n - 1);
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
   if (iters > 0) issue_loads(0);
 
   for (int it = 0; it < iters; ++it) {
-    const int kb0 = k_begin + it * kDecStepKeys + wave * kDecWaveKeys;
+    const int kb0 = (it * p.num_splits + split) * kDecStepKeys + wave * kDecWaveKeys;
     u32x4_t kc[2][4];
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
@@ -408,12 +411,6 @@ __global__ __launch_bounds__(256) void flash_decode_combine_kernel(DecodeParams 
   *reinterpret_cast<u32x2_t *>(p.out + (((size_t)b * p.m + r) * p.H + kvh * p.g + hq) * kRowBytes + d4 * 8) = w;
 }
 
-static int decode_chunk(int n, int num_splits) {
-  int chunk = (n + num_splits - 1) / num_splits;
-  chunk = ((chunk + kDecStepKeys - 1) / kDecStepKeys) * kDecStepKeys;
-  return chunk;
-}
-
 int flash_decode_default_splits(int batch, int n, int kv_head_num) {
   // One workgroup per CU streams best (each keeps 64 KiB of loads in flight and
   // fewer concurrent streams keep the HBM pages open): batch * kv heads * splits
@@ -425,9 +422,7 @@ int flash_decode_default_splits(int batch, int n, int kv_head_num) {
   if (want > cap) want = cap;
   if (want < 1) want = 1;
   if (want > kMaxSplits) want = kMaxSplits;
-  // drop splits that rounding the chunk up to whole steps would leave empty
-  const int chunk = decode_chunk(n, (int)want);
-  return (n + chunk - 1) / chunk;
+  return (int)want;
 }
 
 size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,
@@ -441,8 +436,8 @@ size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_hea
 
 static hipError_t launch_decode_impl(DecodeParams &p, void *workspace, int batch, int kv_head_num, int num_splits,
                                      int dt, bool fused, hipStream_t stream) {
-  p.chunk = decode_chunk(p.n, num_splits);
-  p.num_splits = (p.n + p.chunk - 1) / p.chunk;  // never more than asked for
+  const int nblocks = (p.n + kDecStepKeys - 1) / kDecStepKeys;
+  p.num_splits = num_splits < nblocks ? num_splits : nblocks;  // every split holds at least one block
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
   const size_t slots = (size_t)batch * kv_head_num * p.num_splits * kDecCols;
   p.ws_o = static_cast<float *>(workspace);

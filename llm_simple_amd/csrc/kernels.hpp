@@ -58,5 +58,8 @@ hipError_t launch_add(void *out, const void *lhs, const void *rhs, size_t total,
 // Measurement aid (ceiling_probe.hip): sustained MFMA TFLOP/s of this GPU on N(0,1) bf16 operands,
 // mix 0 = MFMAs alone, mix 1 = MFMAs with the LDS reads and vector instructions of an attention loop.
 hipError_t run_mfma_ceiling(int mix, double target_ms, double *tflops_out);
+hipError_t launch_stream_read(const void *a, const void *b, size_t bytes_each, void *sink, int variant,
+                              hipStream_t stream);
+constexpr size_t kStreamReadSinkBytes = 65536;  // 4 bytes per wave of the largest grid (2 workgroups per CU)
 
 }  // namespace llmhip

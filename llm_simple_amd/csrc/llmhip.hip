@@ -286,6 +286,15 @@ int llmhip_probe_mfma_ceiling(int mix, double target_ms, double *tflops) {
   if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;
   return from_hip(run_mfma_ceiling(mix, target_ms, tflops));
 }
+int llmhip_probe_stream_read(const void *src_a, const void *src_b, size_t bytes_each, void *sink, size_t sink_bytes,
+                             int variant, void *stream) {
+  if (!src_a || !src_b || !sink || bytes_each == 0 || bytes_each % 16 != 0 || (variant != 0 && variant != 1))
+    return LLMHIP_ERR_INVALID_ARG;
+  if (sink_bytes < kStreamReadSinkBytes) return LLMHIP_ERR_WORKSPACE;
+  if (!all_aligned16(src_a, src_b, sink)) return LLMHIP_ERR_INVALID_ARG;
+  if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;
+  return from_hip(launch_stream_read(src_a, src_b, bytes_each, sink, variant, static_cast<hipStream_t>(stream)));
+}
 int llmhip_set_device(int device) {
   if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;
   return from_hip(hipSetDevice(device));

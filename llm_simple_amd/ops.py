@@ -42,6 +42,7 @@ SYMBOLS = {
     "llmhip_device_count": (_i, []),
     "llmhip_device_props": (_i, [_i, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_sz)]),
     "llmhip_probe_mfma_ceiling": (_i, [_i, ctypes.c_double, ctypes.POINTER(ctypes.c_double)]),
+    "llmhip_probe_stream_read": (_i, [_vp, _vp, _sz, _vp, _sz, _i, _vp]),
     "llmhip_set_device": (_i, [_i]),
     "llmhip_malloc": (_i, [ctypes.POINTER(_vp), _sz]),
     "llmhip_free": (_i, [_vp]),
@@ -235,6 +236,19 @@ def probe_mfma_ceiling(mix, target_ms=60.0):
     t = ctypes.c_double(0.0)
     _check(lib.llmhip_probe_mfma_ceiling(mix, float(target_ms), ctypes.byref(t)), "probe_mfma_ceiling")
     return t.value
+
+
+STREAM_READ_SINK_BYTES = 65536
+
+
+def probe_stream_read(a, b, sink, variant, stream=None):
+    """Enqueues a plain streaming read of the two equally sized device tensors a and b (a measurement aid:
+    what a kernel that only reads gets from the memory system)."""
+    nbytes = a.numel() * a.element_size()
+    if b.numel() * b.element_size() != nbytes:
+        raise ValueError("probe_stream_read: a and b must have the same size")
+    _check(lib.llmhip_probe_stream_read(_ptr(a), _ptr(b), nbytes, _ptr(sink), sink.numel() * sink.element_size(),
+                                        variant, stream), "probe_stream_read")
 
 
 def _bf16_round_trip(x):

@@ -5,16 +5,20 @@
 // softmax row per head over the whole contiguous KV cache
 // [max_seq_len][Hkv][128] (src/llama2_layer_npu.cpp:1148-1149).  That is a
 // pure stream of K and V through the chip, so the kernel is organised around
-// HBM: grid = (KV split, kv head, sequence); each workgroup owns a contiguous
-// run of keys of one kv head, each of its 4 waves takes 32 keys per step, and
-// K and V of every key are read from HBM exactly once for all group_size query
-// heads (and all m <= 16/group_size query rows) that share the kv head.
+// HBM: grid = (KV split, kv head, sequence); a workgroup takes every
+// num_splits-th block of 128 keys of one kv head (the workgroups of a sequence
+// walk through its cache side by side), each of its 4 waves 32 keys of a block,
+// and K and V of every key are read from HBM exactly once for all group_size
+// query heads (and all m <= 16/group_size query rows) that share the kv head.
 //
 // The m*group_size query rows are the 16 columns of mfma_f32_16x16x32
-// (S^T = K Q^T, O^T += V^T P^T); unused columns are zero.  K fragments go from
-// global memory straight into the A-operand layout (64 contiguous bytes per
-// 4 lanes); V is staged in a wave-private LDS region and read transposed with
-// ds_read_b64_tr_b16.  Each wave keeps its own running (max, sum, O); the four
+// (S^T = K Q^T, O^T += V^T P^T); unused columns are zero.  Every load
+// instruction fetches whole 256-byte head rows (16 lanes per row); K and V are
+// staged in wave-private LDS regions, K read back in the A-operand layout
+// (loading K straight into that layout -- 16 rows x 16 bytes per quarter wave --
+// costs the texture cache 16 tag look-ups where this costs 2, and measured 1-2 %
+// slower), V read transposed with ds_read_b64_tr_b16.  Each wave keeps its own
+// running (max, sum, O); the four
 // waves are merged through LDS at the end and the workgroup writes either the
 // final rows (one split) or an fp32 partial (max, sum, unnormalised O) that
 // flash_decode_combine_kernel folds with the log-sum-exp rule.  (Folding inside
@@ -38,7 +42,7 @@ constexpr int kDecThreads = 256;
 constexpr int kDecWaveKeys = 32;                  // keys per wave per step
 constexpr int kDecStepKeys = 4 * kDecWaveKeys;    // keys per workgroup per step
 constexpr int kDecCols = 16;                      // query rows per kv head (MFMA N)
-constexpr int kDecWaveLds = kDecWaveKeys * kRowBytes;  // 8 KiB V staging per wave
+constexpr int kDecWaveLds = kDecWaveKeys * kRowBytes;  // 8 KiB of staging per wave, for K and for V
 
 struct DecodeParams {
   const char *q;
@@ -115,7 +119,7 @@ __device__ __forceinline__ int v_swizzle32_off(int row, int granule) {
 template <typename T, bool FUSED>
 __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams p) {
   using E = Elem<T>;
-  __shared__ __attribute__((aligned(16))) char lds[4 * kDecWaveLds + 4 * kDecCols * 2 * 4];
+  __shared__ __attribute__((aligned(16))) char lds[8 * kDecWaveLds];
 
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -157,17 +161,17 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
   float m_run = -INFINITY, l_run = 0.0f;
 
   char *vl = lds + wave * kDecWaveLds;
+  char *kl = lds + (4 + wave) * kDecWaveLds;
 
-  u32x4_t kn[2][4], vn[8];
+  u32x4_t kn[8], vn[8];
   auto issue_loads = [&](int it) {
     const int kb0 = (it * p.num_splits + split) * kDecStepKeys + wave * kDecWaveKeys;
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-      const int key = min(kb0 + blk * 16 + col, p.n - 1);
-      const char *kp = kbase + (size_t)key * kv_row_bytes + cg * 16;
-      if (FUSED && key == p.fused_pos) kp = p.new_k + (size_t)kvh * kRowBytes + cg * 16;
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) kn[blk][kk] = global_load_b128(kp + kk * 64);
+    for (int i = 0; i < 8; ++i) {
+      const int key = min(kb0 + 4 * i + cg, p.n - 1);
+      const char *kp = kbase + (size_t)key * kv_row_bytes + col * 16;
+      if (FUSED && key == p.fused_pos) kp = p.new_k + (size_t)kvh * kRowBytes + col * 16;
+      kn[i] = global_load_b128(kp);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -183,12 +187,10 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
   for (int it = 0; it < iters; ++it) {
     const int kb0 = (it * p.num_splits + split) * kDecStepKeys + wave * kDecWaveKeys;
     u32x4_t kc[2][4];
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) kc[blk][kk] = kn[blk][kk];
-    // stage V (rows 4i+cg, granule col) in this wave's LDS region
+    // stage K and V (rows 4i+cg, granule col) in this wave's LDS regions
     __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lds_write_b128(kl, (4 * i + cg) * kRowBytes + ((col ^ ((4 * i + cg) & 15)) << 4), kn[i]);
 #pragma unroll
     for (int i = 0; i < 8; ++i) lds_write_b128(vl, v_swizzle32_off(4 * i + cg, col), vn[i]);
     if (FUSED && kb0 < k_end) {  // the new token's V row goes to the cache (vn is refilled below)
@@ -201,6 +203,12 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
     }
     __builtin_amdgcn_wave_barrier();
     if (it + 1 < iters) issue_loads(it + 1);
+    // K fragments (A operand): key blk*16+col, dims 32kk + 8cg .. +7
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk)
+        kc[blk][kk] = lds_read_b128(kl, (blk * 16 + col) * kRowBytes + (((4 * kk + cg) ^ col) << 4));
 
     if (kb0 < k_end) {
       if (FUSED) {
@@ -281,7 +289,7 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
   l_tot += xor_lane(l_tot, 32);
   __syncthreads();
   float *lo_f = reinterpret_cast<float *>(lds);                      // [wave][col][128]
-  float *lml = reinterpret_cast<float *>(lds + 4 * kDecWaveLds);     // [wave][col][2]
+  float *lml = reinterpret_cast<float *>(lds + 4 * kDecWaveLds);     // [wave][col][2] (the K staging space)
 #pragma unroll
   for (int d = 0; d < 8; ++d)
     *reinterpret_cast<f32x4_t *>(lo_f + ((wave * kDecCols + col) * kHeadDim + 16 * d + 4 * cg)) = o[d];

@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
   char *kl = lds + (4 + wave) * kDecWaveLds;
 
   u32x4_t kn[8], vn[8];
-  auto issue_loads = [&](int it) {
+  auto issue_k = [&](int it) {
     const int kb0 = (it * p.num_splits + split) * kDecStepKeys + wave * kDecWaveKeys;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -173,6 +173,9 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
       if (FUSED && key == p.fused_pos) kp = p.new_k + (size_t)kvh * kRowBytes + col * 16;
       kn[i] = global_load_b128(kp);
     }
+  };
+  auto issue_v = [&](int it) {
+    const int kb0 = (it * p.num_splits + split) * kDecStepKeys + wave * kDecWaveKeys;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int key = min(kb0 + 4 * i + cg, p.n - 1);
@@ -182,27 +185,24 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
     }
   };
 
-  if (iters > 0) issue_loads(0);
+  // K and V of a step are fetched one after the other, each while the other half of the step is
+  // computed: a wave has 8 KiB of loads in flight at any time, the CU 32 KiB.  That is where this
+  // memory system streams fastest -- with both in flight together (64 KiB per CU) every large shape
+  // measured 2-3 % slower, and a plain read kernel shows the same optimum.
+  // (The first step's K and V start together: one memory round trip less for a workgroup with one step.)
+  if (iters > 0) {
+    issue_k(0);
+    issue_v(0);
+  }
 
   for (int it = 0; it < iters; ++it) {
     const int kb0 = (it * p.num_splits + split) * kDecStepKeys + wave * kDecWaveKeys;
     u32x4_t kc[2][4];
-    // stage K and V (rows 4i+cg, granule col) in this wave's LDS regions
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int i = 0; i < 8; ++i) lds_write_b128(kl, (4 * i + cg) * kRowBytes + ((col ^ ((4 * i + cg) & 15)) << 4), kn[i]);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) lds_write_b128(vl, v_swizzle32_off(4 * i + cg, col), vn[i]);
-    if (FUSED && kb0 < k_end) {  // the new token's V row goes to the cache (vn is refilled below)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int key = min(kb0 + 4 * i + cg, p.n - 1);
-        if (key == p.fused_pos)
-          *reinterpret_cast<u32x4_t *>(const_cast<char *>(vbase) + (size_t)key * kv_row_bytes + col * 16) = vn[i];
-      }
-    }
     __builtin_amdgcn_wave_barrier();
-    if (it + 1 < iters) issue_loads(it + 1);
+    if (it > 0) issue_v(it);
     // K fragments (A operand): key blk*16+col, dims 32kk + 8cg .. +7
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
@@ -268,6 +268,19 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
       psum = dot2_ones<T>(pf[3], psum);
       l_run = l_run * alpha + psum;
       // ---- O^T += V^T P^T ----
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int i = 0; i < 8; ++i) lds_write_b128(vl, v_swizzle32_off(4 * i + cg, col), vn[i]);
+      if (FUSED) {  // the new token's V row goes to the cache
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int key = min(kb0 + 4 * i + cg, p.n - 1);
+          if (key == p.fused_pos)
+            *reinterpret_cast<u32x4_t *>(const_cast<char *>(vbase) + (size_t)key * kv_row_bytes + col * 16) = vn[i];
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      if (it + 1 < iters) issue_k(it + 1);
       const int vr = 4 * cg + (col >> 2);
       const int sub = (col & 1) * 8;
 #pragma unroll
@@ -281,6 +294,8 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
         for (int i = 0; i < 4; ++i) acc[i] *= alpha;
         o[d] = E::mfma16(vf, pf, acc);
       }
+    } else if (it + 1 < iters) {
+      issue_k(it + 1);
     }
   }
 

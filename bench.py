@@ -293,6 +293,10 @@ def bench_rope_append(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
     settle(torch, step, warmup)
     ms, _, _ = timed(torch, timer, step, max(steps, MIN_REPS))
     nbytes = 2 * S * 128 * (2 * H + 4 * Hkv) + S * 64 * 8
+    # a device-to-device copy that moves the same number of bytes (half read, half written), timed the same way
+    src = torch.empty(nbytes // 2, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    copy_ms, _, _ = timed(torch, timer, lambda _: dst.copy_(src), max(steps, MIN_REPS))
     # bit-exact against the oracle on the first and last 32 tokens
     from oracle import oracle as orc
     tab = table.cpu().numpy()
@@ -302,7 +306,8 @@ def bench_rope_append(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
         bad += int(np.count_nonzero(host_bits(oq[sl]) != orc.rope(host_bits(q[sl]), tab, lo, True, DT_BF16)))
         bad += int(np.count_nonzero(host_bits(kc[sl]) != orc.rope(host_bits(k[sl]), tab, lo, True, DT_BF16)))
         bad += int(np.count_nonzero(host_bits(vc[sl]) != host_bits(v[sl])))
-    return {"S": S, "ms": ms, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9, "mismatched_elements": bad}
+    return {"S": S, "ms": ms, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9, "mismatched_elements": bad,
+            "ms_plain_copy": copy_ms, "gbs_plain_copy": nbytes / (copy_ms * 1e-3) / 1e9}
 
 
 def bench_attention_block(ops, torch, timer, S, steps, warmup, H=28, Hkv=4):
@@ -496,12 +501,14 @@ def main():
 
     if "rope" in legs:
         r = bench_rope_append(ops, torch, timer, args.seq, args.steps, args.warmup)
-        log(f"rope+append S={args.seq}: {r['ms'] * 1e3:.1f} us {r['gbs']:.0f} GB/s")
+        log(f"rope+append S={args.seq}: {r['ms'] * 1e3:.1f} us {r['gbs']:.0f} GB/s; a device-to-device copy moving the "
+            f"same bytes: {r['ms_plain_copy'] * 1e3:.1f} us {r['gbs_plain_copy']:.0f} GB/s")
         extra["rope_kv_append"] = {"S": r["S"], "us": r["ms"] * 1e3, "gbs": r["gbs"],
                                    "frac": r["gbs"] / PEAK_HBM_GBS,
                                    "traffic": MEASURED_TRAFFIC_BYTES.get(("rope", r["S"])),
                                    "traffic_source": TRAFFIC_SOURCE,
-                                   "mismatched_elements": r["mismatched_elements"]}
+                                   "mismatched_elements": r["mismatched_elements"],
+                                   "us_plain_copy": r["ms_plain_copy"] * 1e3, "gbs_plain_copy": r["gbs_plain_copy"]}
 
     if "block" in legs:
         r = bench_attention_block(ops, torch, timer, args.seq, args.steps // 8, 3)

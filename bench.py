@@ -42,9 +42,9 @@ DT_BF16 = 5
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE summaries under profiles/ (not measured in this run)"
 MEASURED_TRAFFIC_BYTES = {
     ("prefill", 4096): (47179 + 28672) * 1024,             # algorithmic 65536 KiB
-    ("decode", 16, 32768): (2097572 + 656) * 1024,         # algorithmic 2097152 KiB
-    ("decode", 1, 32768): (131250 + 656) * 1024,           # algorithmic 131072 KiB
-    ("rope", 4096): (40527 + 36864) * 1024,                # algorithmic 75776 KiB
+    ("decode", 16, 32768): (2097637 + 656) * 1024,         # algorithmic 2097152 KiB
+    ("decode", 1, 32768): (131317 + 656) * 1024,           # algorithmic 131072 KiB
+    ("rope", 4096): (40753 + 36864) * 1024,                # algorithmic 75776 KiB
     ("chunked", 256, 33024): (136014 + 33557 + 33339 + 1792) * 1024,   # prefill kernel + combine
     ("chunked", 40, 131072): (524998 + 26241 + 26437 + 400) * 1024,
 }
@@ -412,7 +412,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--seq", type=int, default=4096, help="prefill sequence length of the timed step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: ceiling,prefill,chunked,decode,rope,block (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs: ceiling,prefill,chunked,decode,decode_step,rope,block (default all)")
     ap.add_argument("--decode-shapes", default="16x32768,1x32768,1x4096,1x16384,16x4096,16x16384",
                     help="comma list of BATCHxKVLEN decode cases; the first one is the headline")
     ap.add_argument("--chunk-shapes", default="256x33024x28x4,40x131072x40x8",
@@ -434,7 +434,7 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     timer = HipTimer(ops.lib)
-    legs = set(args.only.split(",")) if args.only else {"ceiling", "prefill", "chunked", "decode", "rope", "block"}
+    legs = set(args.only.split(",")) if args.only else {"ceiling", "prefill", "chunked", "decode", "decode_step", "rope", "block"}
     legs.discard("none")
     extra = {}
 
@@ -504,17 +504,19 @@ def main():
                                   "(llmhip_probe_stream_read)"},
             "workload": f"Qwen2.5-32B decode bf16 H=40 Hkv=8 n={head['n']} batch={head['batch']} "
                         f"({head['kv_bytes'] / 2 ** 20:.0f} MiB of K+V per launch, cold)"}
-        extra["decode_step"] = [bench_decode_step(ops, torch, timer, n, args.steps, args.warmup) for n in (4096, 32768)]
-        for r in extra["decode_step"]:
-            log(f"decode step B=1 n={r['n']}: rope+append, decode, combine {r['us_three_launches']:.1f} us; fused into the "
-                f"decode kernel {r['us_fused']:.1f} us ({r['kv_gbs_fused']:.0f} GB/s), bit-identical {r['fused_output_bit_identical']}")
-        torch.cuda.empty_cache()
         extra["decode_all"] = [
             {"batch": r["batch"], "n": r["n"], "splits": r["splits"], "us_cold": r["ms_cold"] * 1e3,
              "gbs_cold": r["gbs_cold"], "frac_cold": r["gbs_cold"] / PEAK_HBM_GBS,
              "us_hot": r["ms_hot"] * 1e3, "gbs_hot": r["gbs_hot"], "max_abs_err": r["max_abs_err"],
              "us_plain_read": r["ms_plain_read"] * 1e3, "frac_of_plain_read": r["ms_plain_read"] / r["ms_cold"]}
             for r in dec]
+
+    if "decode_step" in legs:
+        extra["decode_step"] = [bench_decode_step(ops, torch, timer, n, args.steps, args.warmup) for n in (4096, 32768)]
+        for r in extra["decode_step"]:
+            log(f"decode step B=1 n={r['n']}: rope+append, decode, combine {r['us_three_launches']:.1f} us; fused into the "
+                f"decode kernel {r['us_fused']:.1f} us ({r['kv_gbs_fused']:.0f} GB/s), bit-identical {r['fused_output_bit_identical']}")
+        torch.cuda.empty_cache()
 
     if "rope" in legs:
         r = bench_rope_append(ops, torch, timer, args.seq, args.steps, args.warmup)

@@ -454,10 +454,11 @@ template <int NW> struct DirectLoader {
 // Every wave runs S(j+1) = K Q^T, the softmax of tile j and P(j).V(j) as one instruction
 // stream (the compiler interleaves the softmax VALU work with the MFMAs); the tile loads
 // are spread over that stream.  NW = 4: two workgroups per CU (small problems); NW = 8:
-// one workgroup per CU, K/V tiles shared by 256 rows.  KB = 1 (with NW = 8): 128 rows, every row
-// block worked on by two waves that each take one 32-key half of every tile and are merged
-// through LDS at the end -- for sequences so short that there is at most about one 128-row
-// workgroup per CU, where the serial MFMA chain of a wave is what the launch waits for.
+// one workgroup per CU, K/V tiles shared by 256 rows.  KB = 1: every row block worked on by two
+// waves that each take one 32-key half of every tile and are merged through LDS at the end (NW = 8:
+// 128 rows; NW = 4: 64 rows, two workgroups per CU) -- for sequences so short that there is at most
+// about one 128-row workgroup per CU, where the serial MFMA chain of a wave is what the launch
+// waits for.
 // ---------------------------------------------------------------------------
 template <typename T, int NW, int KB>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel(PrefillParams p) {
@@ -553,10 +554,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
         w.mask(s_cur, key0, qtok, offset_, n_);
       // a burst of loads would stall every wave behind the texture addresser's queue:
       // one load every 8 * KB / PER MFMAs instead
+      // (Paired waves, KB == 1, run short sequences, where a step is shorter than a memory round
+      // trip: there all loads of a step go out with its first MFMAs.)
       auto k_hook = [&](int i) {
 #pragma unroll
-        for (int r = 0; r < PER; ++r)
-          if (i == (8 * KB / PER) * r + 1) ld.template issue<false>(kbase, jk, kslot * kTileBytes, r);
+        for (int r = 0; r < PER; ++r) {
+          if (KB == 1) {
+            if (i == r) ld.template issue<false>(kbase, jk, kslot * kTileBytes, r);
+            if (i == PER + r) ld.template issue<true>(vbase, jv, kVRegion + vslot * kTileBytes, r);
+          } else if (i == (8 * KB / PER) * r + 1) {
+            ld.template issue<false>(kbase, jk, kslot * kTileBytes, r);
+          }
+        }
       };
       // The MFMAs of S(j+1) overlap the softmax of tile j: the first ones run beside the row
       // maximum chain, the rest -- and the MFMAs of P.V -- beside the exponentials.  (For the
@@ -570,7 +579,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
       w.pv(lds, slot * kTileBytes, [&](int i) {
 #pragma unroll
         for (int r = 0; r < PER; ++r)
-          if (i == (8 * KB / PER) * r + 1)
+          if (KB != 1 && i == (8 * KB / PER) * r + 1)
             ld.template issue<true>(vbase, jv, kVRegion + vslot * kTileBytes, r);
       });
     } else {
@@ -724,7 +733,8 @@ static int device_compute_units() {
 // never split: the fp32 partials would cost more HBM traffic than K and V themselves.
 struct PrefillPlan {
   bool rows256, pack;
-  bool pair;  // 128-row workgroups of 8 waves, two waves per row block (short sequences)
+  bool pair;  // two waves per row block, each on one 32-key half of every tile (short sequences)
+  bool rows64;  // with pair: 64-row workgroups of 4 waves, two per CU, instead of 128 rows and 8 waves
   int num_splits, chunk;
 };
 static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cus) {
@@ -737,13 +747,18 @@ static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cu
   // the most keys, so two waves share every row block (measured at H=28, bf16, 256 CUs, 4-wave /
   // paired 8-wave workgroups, us: S=1024 22.6/20.2, S=1536 32.8/27.9, S=2048 45.6/42.1,
   // S=2560 60.8/64.6, S=3072 76.3/86.0)
-  pl.pair = !pl.rows256 && (long long)((m + 127) / 128) * H <= 2LL * cus;
+  const long long wg128 = (long long)((m + 127) / 128) * H;
+  pl.pair = !pl.rows256 && wg128 <= 2LL * cus;
+  // Up to about 1.2 such workgroups per CU, halves of them (64 rows, 4 waves, two resident per CU) finish
+  // sooner: the heavy tiles meet less competition for their SIMDs (128-row / 64-row, us: S=256
+  // 10.5/8.6, S=512 13.6/11.5, S=1024 20.2/17.8, S=1280 25.4/23.9, S=1408 27.9/27.5, S=1536 28.0/29.4)
+  pl.rows64 = pl.pair && 5 * wg128 <= 6LL * cus;
   pl.num_splits = 1;
   pl.chunk = 0x7fffffc0;
   const long long n_vis = ((long long)m + offset < n) ? (long long)m + offset : n;  // keys the last row sees
-  if (n_vis < 256) pl.pair = false;
+  if (n_vis < 256) pl.pair = pl.rows64 = false;
   if (pl.rows256 || n_vis < 8LL * m || n_vis < 2048) return pl;
-  pl.pair = false;
+  pl.pair = pl.rows64 = false;
   // Split mode.  A chunk shorter than a 128-row tile packs the g query heads of a kv head into the
   // rows of one tile (K and V of the kv head are then read once, not g times).
   pl.pack = g > 1 && m < 128;
@@ -758,7 +773,8 @@ static PrefillPlan plan_prefill(int m, int n, int offset, int g, int Hkv, int cu
   if (splits <= 1) {
     pl.pack = false;
     pl.rows256 = false;
-    pl.pair = (long long)((m + 127) / 128) * H <= 2LL * cus;
+    pl.pair = wg128 <= 2LL * cus;
+    pl.rows64 = 5 * wg128 <= 6LL * cus;
     return pl;
   }
   long long chunk = (n_vis + splits - 1) / splits;
@@ -797,6 +813,7 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
     pl.chunk = 0x7fffffc0;
     pl.pack = false;
     pl.rows256 = false;
+    pl.rows64 = false;
   }
   p.pack = pl.pack ? 1 : 0;
   p.num_splits = pl.num_splits;
@@ -805,6 +822,8 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
   p.ws_ml = p.ws_o ? p.ws_o + (size_t)pl.num_splits * m * p.H * kHeadDim : nullptr;
   const bool f16 = dt == kDtFloat16;
   if (pl.rows256) return f16 ? launch_prefill_t<_Float16, 8>(p, stream) : launch_prefill_t<__bf16, 8>(p, stream);
+  if (pl.pair && pl.rows64)
+    return f16 ? launch_prefill_t<_Float16, 4, 1>(p, stream) : launch_prefill_t<__bf16, 4, 1>(p, stream);
   if (pl.pair) return f16 ? launch_prefill_t<_Float16, 8, 1>(p, stream) : launch_prefill_t<__bf16, 8, 1>(p, stream);
   return f16 ? launch_prefill_t<_Float16, 4>(p, stream) : launch_prefill_t<__bf16, 4>(p, stream);
 }

@@ -109,3 +109,24 @@ def test_measurement_aids():
     assert 250.0 < mix < alone < 2600.0, (alone, mix)
     cus, mhz, mem = ops.device_props(0)
     assert cus >= 64 and 1000.0 <= mhz <= 3000.0 and mem > (16 << 30)
+
+
+def test_plain_read_probe_reads_every_byte():
+    """llmhip_probe_stream_read XORs everything it reads into one word per wave: the XOR of those words must be
+    the XOR of all 32-bit words of both arrays, for both launch shapes and a size that is not a multiple of the
+    grid's stride."""
+    import torch
+    import llm_simple_amd.ops as ops
+    rng = np.random.default_rng(5)
+    for n_words in (4 * 1000, 4 * 262144 + 4 * 37):
+        a = rng.integers(0, 2 ** 32, n_words, dtype=np.uint32)
+        b = rng.integers(0, 2 ** 32, n_words, dtype=np.uint32)
+        want = int(np.bitwise_xor.reduce(a) ^ np.bitwise_xor.reduce(b))
+        d_a, d_b = to_dev(a.view(np.uint16)), to_dev(b.view(np.uint16))
+        for variant in (0, 1):
+            sink = torch.zeros(ops.STREAM_READ_SINK_BYTES // 4, dtype=torch.int32, device="cuda")
+            ops.probe_stream_read(d_a, d_b, sink, variant)
+            torch.cuda.synchronize()
+            got = int(np.bitwise_xor.reduce(sink.cpu().numpy().view(np.uint32)))
+            assert got == want, (n_words, variant, hex(got), hex(want))
+

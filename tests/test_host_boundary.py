@@ -51,6 +51,15 @@ def test_argument_validation_without_gpu():
     assert lib.llmhip_rope_single(p, p + 4, p, 0, 1, 2, 256, 0, 4, None) == -1
     assert lib.llmhip_rope_kv_append(p, p, p + 6, p, p, p, p, 0, 1, 1, 1, 128, 0, 4, None) == -1
     assert lib.llmhip_flash_decode_gqa_static(p, p, p + 2, p, 1, 16, 16, 5, 8, 128, 1, 5, None) == -1
+    # the plain-read probe: size a multiple of 16, sink of the declared size, aligned pointers
+    assert lib.llmhip_probe_stream_read(p, p, 24, p, ops.STREAM_READ_SINK_BYTES, 0, None) == -1
+    assert lib.llmhip_probe_stream_read(p, p, 32, p, 1024, 0, None) == -3
+    assert lib.llmhip_probe_stream_read(p, p + 4, 32, p, ops.STREAM_READ_SINK_BYTES, 0, None) == -1
+    assert lib.llmhip_probe_stream_read(p, p, 32, p, ops.STREAM_READ_SINK_BYTES, 2, None) == -1
+    # the fused decode step: group size within the kernel's 16 columns, position not negative
+    assert lib.llmhip_decode_step_gqa(p, p, p, p, p, p, p, 0, 17, 1, 128, 0, 5, None) == -2
+    assert lib.llmhip_decode_step_gqa(p, p, p, p, p, p, p, -1, 5, 8, 128, 0, 5, None) == -1
+    assert lib.llmhip_decode_step_gqa(p, p, p + 2, p, p, p, p, 0, 5, 8, 128, 0, 5, None) == -1
     try:
         ops.hip_flash_attn_layer(0, p, p, p, 1, 1, 0, 1, 128, 4)
     except ops.LlmHipError as e:

@@ -43,6 +43,7 @@ constexpr int kDecWaveKeys = 32;                  // keys per wave per step
 constexpr int kDecStepKeys = 4 * kDecWaveKeys;    // keys per workgroup per step
 constexpr int kDecCols = 16;                      // query rows per kv head (MFMA N)
 constexpr int kDecWaveLds = kDecWaveKeys * kRowBytes;  // 8 KiB of staging per wave, for K and for V
+constexpr int kDecLdsPad = 24 * 1024;             // with the 64 KiB of staging: more than half a CU's LDS
 
 struct DecodeParams {
   const char *q;
@@ -362,6 +363,7 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
 // dims per thread, all of a thread's loads issued before any is used), then the 8 groups are merged
 // through LDS.  With few splits the surplus groups have nothing to load.
 constexpr int kMaxSplits = 256;
+constexpr int kDecTargetWgs = 256;  // workgroups of one round: the CUs of the part this is tuned on
 
 template <typename T>
 __global__ __launch_bounds__(256) void flash_decode_combine_kernel(DecodeParams p) {
@@ -434,18 +436,54 @@ __global__ __launch_bounds__(256) void flash_decode_combine_kernel(DecodeParams 
   *reinterpret_cast<u32x2_t *>(p.out + (((size_t)b * p.m + r) * p.H + kvh * p.g + hq) * kRowBytes + d4 * 8) = w;
 }
 
+// Largest split count the default rule considers for batch * kv heads = pairs (any KV length).
+int flash_decode_max_default_splits(long long pairs) {
+  long long base = (kDecTargetWgs + pairs - 1) / pairs;  // one round of workgroups
+  if (base < 8) base = 8;
+  if (base > kMaxSplits) base = kMaxSplits;
+  return (int)base;
+}
+
+// Split count that a simple model of the launch makes fastest.  Workgroups run one per CU in rounds
+// of kDecTargetWgs; a CU of a full round streams 25 GB/s (all of them together what the memory system
+// gives a reader, 6.4 TB/s), a CU of a thin round at most 31 GB/s; a workgroup costs 3 us beyond its
+// bytes, the combine launch 5 us.  Among the counts within 3 % of the best, one that fills its rounds
+// exactly is preferred, else the smallest.  For the common shapes this is about one workgroup per CU
+// (batch 16 x 8 kv heads -> 2 splits, batch 1 -> 32); for pair counts that do not divide a round it
+// finds the count that fills the rounds (model / measured us, n = 8192: batch 12, 1/2/3/5/8 splits ->
+// 138/76/115/75/77 against 133/80/106/76/76; batch 24, 1/2/4 -> 138/163/140 against 150/158/145;
+// batch 40, 1/2/3/4 -> measured 294/242/231/233).
 int flash_decode_default_splits(int batch, int n, int kv_head_num) {
-  // One workgroup per CU streams best (each keeps 64 KiB of loads in flight and
-  // fewer concurrent streams keep the HBM pages open): batch * kv heads * splits
-  // ~ 256, but at least one step (128 keys) of work per split.
   const long long pairs = (long long)batch * kv_head_num;
-  long long want = (256 + pairs - 1) / pairs;
-  long long cap = n / kDecStepKeys;
-  if (cap < 1) cap = 1;
-  if (want > cap) want = cap;
-  if (want < 1) want = 1;
-  if (want > kMaxSplits) want = kMaxSplits;
-  return (int)want;
+  const int nblocks = (n + kDecStepKeys - 1) / kDecStepKeys;
+  int smax = flash_decode_max_default_splits(pairs);
+  if (smax > nblocks) smax = nblocks;
+  if (smax < 1) smax = 1;
+  const double key_bytes = 2.0 * kRowBytes;  // K and V row of one kv head
+  auto model = [&](int s) {
+    const long long wgs = pairs * s;
+    const long long full = wgs / kDecTargetWgs, rest = wgs % kDecTargetWgs;
+    const double wg_bytes = key_bytes * kDecStepKeys * ((nblocks + s - 1) / s);
+    double t = full * (wg_bytes / 25e9 + 3e-6);
+    if (rest > 0) {
+      double rate = 6.4e12 / (double)rest;
+      if (rate > 31e9) rate = 31e9;
+      t += wg_bytes / rate + 3e-6;
+    }
+    return s > 1 ? t + 5e-6 : t;
+  };
+  double t_min = model(1);
+  for (int s = 2; s <= smax; ++s) {
+    const double t = model(s);
+    if (t < t_min) t_min = t;
+  }
+  int first = 0;
+  for (int s = 1; s <= smax; ++s) {
+    if (model(s) > t_min * 1.03) continue;
+    if (first == 0) first = s;
+    if ((pairs * s) % kDecTargetWgs == 0) return s;
+  }
+  return first;
 }
 
 size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,
@@ -466,18 +504,26 @@ static hipError_t launch_decode_impl(DecodeParams &p, void *workspace, int batch
   p.ws_o = static_cast<float *>(workspace);
   p.ws_ml = p.ws_o ? p.ws_o + slots * kHeadDim : nullptr;
   dim3 grid(p.num_splits, kv_head_num, batch);
-  if (dt == kDtFloat16) {
-    if (fused)
-      hipLaunchKernelGGL((flash_decode_kernel<_Float16, true>), grid, dim3(kDecThreads), 0, stream, p);
-    else
-      hipLaunchKernelGGL((flash_decode_kernel<_Float16, false>), grid, dim3(kDecThreads), 0, stream, p);
-  } else {
-    if (fused)
-      hipLaunchKernelGGL((flash_decode_kernel<__bf16, true>), grid, dim3(kDecThreads), 0, stream, p);
-    else
-      hipLaunchKernelGGL((flash_decode_kernel<__bf16, false>), grid, dim3(kDecThreads), 0, stream, p);
+  void (*kern)(DecodeParams) = (dt == kDtFloat16)
+                                   ? (fused ? flash_decode_kernel<_Float16, true> : flash_decode_kernel<_Float16, false>)
+                                   : (fused ? flash_decode_kernel<__bf16, true> : flash_decode_kernel<__bf16, false>);
+  // kDecLdsPad bytes of dynamic LDS that nobody touches keep a second workgroup off the CU (two of
+  // them would put 64 KiB of loads in flight again).  More than 64 KiB of LDS in total is an opt-in
+  // per device and kernel.
+  static std::atomic<uint64_t> attr_done[4] = {};
+  const int which = (dt == kDtFloat16 ? 0 : 2) + (fused ? 1 : 0);
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (!(attr_done[which].load(std::memory_order_acquire) & bit)) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kDecLdsPad);
+    if (e != hipSuccess) return e;
+    attr_done[which].fetch_or(bit, std::memory_order_release);
   }
-  hipError_t e = hipGetLastError();
+  hipLaunchKernelGGL(kern, grid, dim3(kDecThreads), kDecLdsPad, stream, p);
+  e = hipGetLastError();
   if (e != hipSuccess || p.num_splits == 1) return e;
   dim3 cgrid(p.rows, kv_head_num, batch);
   if (dt == kDtFloat16)

@@ -20,6 +20,7 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
 size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,
                                     int num_splits);
 int flash_decode_default_splits(int batch, int n, int kv_head_num);
+int flash_decode_max_default_splits(long long pairs);
 hipError_t launch_flash_decode(void *out, const void *q, const void *k, const void *v,
                                void *workspace, int batch, int m, int n, int offset,
                                int64_t kv_seq_stride, int group_size, int kv_head_num,

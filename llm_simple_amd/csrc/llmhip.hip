@@ -150,9 +150,8 @@ size_t llmhip_flash_decode_workspace_bytes(int batch, int group_size, int kv_hea
                                            int head_dim, int num_splits) {
   if (batch < 1 || group_size < 1 || kv_head_num < 1 || head_dim != 128) return 0;
   if (num_splits <= 0) {
-    // the largest count the default rule picks for any KV length: ceil(256 / (batch * kv heads))
-    const long long pairs = (long long)batch * kv_head_num;
-    num_splits = (int)((256 + pairs - 1) / pairs);
+    // the largest count the default rule picks for any KV length
+    num_splits = flash_decode_max_default_splits((long long)batch * kv_head_num);
   }
   if (num_splits > kMaxDecodeSplits) num_splits = kMaxDecodeSplits;
   return flash_decode_workspace_bytes(batch, 1, group_size, kv_head_num, num_splits);

@@ -120,10 +120,10 @@ int llmhip_flash_decode_default_splits(int batch, int n, int kv_head_num);
  * `workspace`: the split-KV partials go to a fixed array of
  * llmhip_flash_decode_static_scratch_bytes() (4 MiB) of device memory inside the library, which
  * every GPU the library runs on holds until the process ends.  The call allocates and frees
- * nothing.  Limit: batch * kv_head_num * num_splits * 8320 bytes must fit the array (504 slots,
- * e.g. the default split count for any batch * kv_head_num <= 252); larger requests are rejected
- * with LLMHIP_ERR_WORKSPACE before anything is launched (one split needs no scratch and always
- * fits).  All calls on a GPU share the array: calls that overlap on one GPU (different streams,
+ * nothing.  Limit: batch * kv_head_num * num_splits * 8320 bytes must fit the array (504 slots);
+ * an explicit num_splits beyond that is rejected with LLMHIP_ERR_WORKSPACE before anything is
+ * launched, the default count (num_splits <= 0) is lowered until it fits (one split needs no
+ * scratch and always fits).  All calls on a GPU share the array: calls that overlap on one GPU (different streams,
  * different threads) race; calls on one stream are ordered and safe. */
 int llmhip_flash_decode_gqa_static(void *out, const void *q, const void *k_cache,
                                    const void *v_cache, int batch, int n, int64_t kv_seq_stride,

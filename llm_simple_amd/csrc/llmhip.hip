@@ -188,7 +188,13 @@ int llmhip_flash_decode_gqa_static(void *out, const void *q, const void *k_cache
   if (!dtype_ok(dt)) return LLMHIP_ERR_INVALID_ARG;
   if (head_dim != 128 || group_size > kMaxDecodeCols) return LLMHIP_ERR_UNSUPPORTED;
   if (batch > 65535 || kv_head_num > 65535) return LLMHIP_ERR_UNSUPPORTED;
-  if (num_splits <= 0) num_splits = flash_decode_default_splits(batch, n, kv_head_num);
+  if (num_splits <= 0) {
+    // the default count, lowered until its partials fit the fixed array (one split needs none)
+    num_splits = flash_decode_default_splits(batch, n, kv_head_num);
+    while (num_splits > 1 &&
+           flash_decode_workspace_bytes(batch, 1, group_size, kv_head_num, num_splits) > kStaticDecodeScratchBytes)
+      --num_splits;
+  }
   if (num_splits > kMaxDecodeSplits) num_splits = kMaxDecodeSplits;
   // the fixed array must hold the partials of every (sequence, kv head, split)
   if (flash_decode_workspace_bytes(batch, 1, group_size, kv_head_num, num_splits) > kStaticDecodeScratchBytes)

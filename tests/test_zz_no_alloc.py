@@ -69,3 +69,29 @@ def test_static_decode_rejects_what_does_not_fit():
     assert lib.llmhip_flash_decode_gqa_static(p, p, p, p, 64, 4096, 4096, 5, 8, 128, 2, DT_BFLOAT16, None) == -3
     assert lib.llmhip_flash_decode_gqa_static(None, p, p, p, 1, 16, 16, 5, 8, 128, 1, DT_BFLOAT16, None) == -1
     assert lib.llmhip_flash_decode_gqa_static(p, p, p, p, 1, 16, 16, 5, 8, 64, 1, DT_BFLOAT16, None) == -2
+
+
+def test_static_decode_lowers_a_default_split_count_that_does_not_fit():
+    """40 sequences x 8 kv heads: the default rule asks for several splits, whose partials would not fit the
+    fixed array; with num_splits <= 0 the call takes the largest count that fits (here one split) and must
+    equal the workspace decode run with that count."""
+    import torch
+    import llm_simple_amd.ops as ops
+    H, Hkv, batch, n, dt = 40, 8, 40, 2048, DT_BFLOAT16
+    g = H // Hkv
+    default = ops.flash_decode_default_splits(batch, n, Hkv)
+    cap = ops.lib.llmhip_flash_decode_static_scratch_bytes()
+    assert default > 1 and ops.flash_decode_workspace_bytes(batch, g, Hkv, 128, default) > cap
+    fits = max(s for s in range(1, default) if ops.flash_decode_workspace_bytes(batch, g, Hkv, 128, s) <= cap)
+    q = normal_bits(61, (batch, 1, H, 128), dt)
+    k = normal_bits(62, (batch, n, Hkv, 128), dt)
+    v = normal_bits(63, (batch, n, Hkv, 128), dt)
+    dq, dk, dv = to_dev(q), to_dev(k), to_dev(v)
+    wsb = ops.flash_decode_workspace_bytes(batch, g, Hkv, 128, fits)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
+    want, got = dev_empty(q.shape), dev_empty(q.shape)
+    ops.hip_flash_decode_gqa_layer(want, dq, dk, dv, ws, wsb, batch, n, n, g, Hkv, 128, fits, dt)
+    ops.hip_flash_decode_gqa_static_layer(got, dq, dk, dv, batch, n, n, g, Hkv, 128, 0, dt)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(got), to_host(want))
+

@@ -31,24 +31,6 @@ namespace llmhip {
 
 constexpr int kRopeUnits = 2;  // 32-byte units per thread, a grid apart: twice the loads in flight per wave
 
-// n / d for 32-bit n by multiply and shift (Granlund-Montgomery, round-up variant): exact for every n.
-struct FastDiv {
-  uint32_t d, m, l;  // l = ceil(log2 d); m = floor(2^32 (2^l - d) / d) + 1
-};
-static FastDiv make_fast_div(uint32_t d) {
-  FastDiv f;
-  f.d = d;
-  f.l = 0;
-  while ((1ull << f.l) < d) ++f.l;
-  f.m = (uint32_t)((((1ull << f.l) - d) << 32) / d + 1);
-  return f;
-}
-__device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv &f) {
-  if (f.l == 0) return n;  // d == 1
-  const uint32_t t = (uint32_t)(((uint64_t)n * f.m) >> 32);
-  return (t + ((n - t) >> 1)) >> (f.l - 1);
-}
-
 struct RopeParams {
   const char *in_q, *in_k, *in_v;
   char *out_q, *out_k, *out_v;

@@ -172,7 +172,7 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
       const int key = min(kb0 + 4 * i + cg, p.n - 1);
       const char *kp = kbase + (size_t)key * kv_row_bytes + col * 16;
       if (FUSED && key == p.fused_pos) kp = p.new_k + (size_t)kvh * kRowBytes + col * 16;
-      kn[i] = global_load_b128(kp);
+      kn[i] = global_load_b128_nt(kp);
     }
   };
   auto issue_v = [&](int it) {
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
       const int key = min(kb0 + 4 * i + cg, p.n - 1);
       const char *vp = vbase + (size_t)key * kv_row_bytes + col * 16;
       if (FUSED && key == p.fused_pos) vp = p.new_v + (size_t)kvh * kRowBytes + col * 16;
-      vn[i] = global_load_b128(vp);
+      vn[i] = global_load_b128_nt(vp);
     }
   };
 

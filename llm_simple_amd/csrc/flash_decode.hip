@@ -17,8 +17,11 @@
 // staged in wave-private LDS regions, K read back in the A-operand layout
 // (loading K straight into that layout -- 16 rows x 16 bytes per quarter wave --
 // costs the texture cache 16 tag look-ups where this costs 2, and measured 1-2 %
-// slower), V read transposed with ds_read_b64_tr_b16.  Each wave keeps its own
-// running (max, sum, O); the four
+// slower), V read transposed with ds_read_b64_tr_b16.  K and V are read once, so
+// their loads are non-temporal (7.1 TB/s at 2 GiB where ordinary loads give 6.2),
+// and K and V of a step are fetched one after the other so that a CU has 32 KiB
+// in flight, not 64 (see the loop).  Each wave keeps its own running (max, sum,
+// O); the four
 // waves are merged through LDS at the end and the workgroup writes either the
 // final rows (one split) or an fp32 partial (max, sum, unnormalised O) that
 // flash_decode_combine_kernel folds with the log-sum-exp rule.  (Folding inside
@@ -30,7 +33,8 @@
 // 33.4 us, and 15.0 us against 10.6 us at 4096 keys: the chain store-acknowledge, atomic,
 // two dependent rounds of memory-latency loads in ONE workgroup is longer than a launch.
 // Eight-wave workgroups, half as many, merging pairs of splits through LDS: 4.5 TB/s
-// against 6.0 -- a CU draws about 35 GB/s however many waves ask, so all 256 must stream.)
+// against 6.0 at the time -- a CU draws about 31-35 GB/s however many waves ask, so all of
+// them must stream.)
 #include <atomic>
 
 #include "common.hpp"

@@ -13,6 +13,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include <vector>
 
 #include "common.hpp"
@@ -125,16 +127,16 @@ uint16_t normal_bf16(uint64_t i) {
 // per CU, 4 in flight (best below).  sink: 4 bytes per wave of the grid.
 hipError_t launch_stream_read(const void *a, const void *b, size_t bytes_each, void *sink, int variant,
                               hipStream_t stream) {
-  static int cus_of[64] = {};  // per device; written once with the same value by whoever comes first
+  static std::atomic<int> cus_of[64];  // per device; every writer stores the same value
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
-  int cus = cus_of[dev];
-  if (cus == 0) {
+  int cus = cus_of[dev].load(std::memory_order_relaxed);
+  if (cus <= 0) {
     e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess || cus <= 0) return e != hipSuccess ? e : hipErrorInvalidDevice;
-    cus_of[dev] = cus;
+    cus_of[dev].store(cus, std::memory_order_relaxed);
   }
   const u32x4_t *pa = static_cast<const u32x4_t *>(a), *pb = static_cast<const u32x4_t *>(b);
   unsigned *ps = static_cast<unsigned *>(sink);

@@ -44,6 +44,9 @@ def ulp(x, dt):
     return 2.0 ** (np.floor(np.log2(ax)) - mant)
 
 
+BF16_LAYER_STATS = []  # (elements, beyond two steps, beyond three steps) of every bf16 comparison made
+
+
 def check_attention(out_bits, q, k, v, n, offset, dt, batch=None, layer_style=True):
     """Compare HIP output bits with both oracles.
 
@@ -54,7 +57,7 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None, layer_style=Tr
     per million; bf16 (no reference code, the same chain with bf16 casts, which by itself
     sits up to ~1.2e-2 from the fp32 oracle on rows that see few keys,
     tests/test_oracle_attention.py) within TOL or two steps for all but 200 elements per
-    million and within TOL or three steps for all but 2 per million.  layer_style=False skips the second
+    million and within TOL or three steps for all but 5 per million (at least 4 elements).  layer_style=False skips the second
     comparison: for scores of magnitude ~30 the layer-style chain's rounding of the scores to
     fp16 alone (steps of 2^-6) moves the probabilities by more than TOL."""
     got = orc.widen(out_bits, dt)
@@ -80,9 +83,11 @@ def check_attention(out_bits, q, k, v, n, offset, dt, batch=None, layer_style=Tr
         assert off <= max(1, got.size // 10 ** 6), f"{off} elements off the layer-style oracle, worst {d16.max()}"
     else:
         # bf16: the layer-style chain rounds scores and probabilities to 8 bits, so single elements of rows
-        # that see few keys land a step or two further away (measured on the kernels over 27 shapes: at most
-        # 76 per million beyond TOL-or-2-steps, at most 0.3 per million beyond TOL-or-3-steps)
+        # that see few keys land a step or two further away (measured on the kernels over 27 benchmark-like
+        # and 229 random shapes: at most 76 per million beyond TOL-or-2-steps; beyond TOL-or-3-steps at most
+        # 2 elements of any output below a million elements and 0.3 per million above)
         off2, off3 = near(2), near(3)
+        BF16_LAYER_STATS.append((got.size, off2, off3))
         assert off2 <= max(4, got.size * 200 // 10 ** 6), f"{off2} of {got.size} elements beyond 2 steps, worst {d16.max()}"
-        assert off3 <= max(2, got.size * 2 // 10 ** 6), f"{off3} of {got.size} elements beyond 3 steps, worst {d16.max()}"
+        assert off3 <= max(4, got.size * 5 // 10 ** 6), f"{off3} of {got.size} elements beyond 3 steps, worst {d16.max()}"
     return e32, float(d16.max())

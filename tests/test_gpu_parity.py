@@ -456,6 +456,46 @@ def test_flash_decode_random_shapes():
         check_attention(to_host(d_out), q, k, v, n, n - 1, dt, batch=True)
 
 
+def test_attention_random_shapes():
+    """Seeded sweep of the reference-signature attention entry point over the four regimes of its dispatch:
+    square causal prefill (all kernel shapes for short sequences), a chunk of few rows over a long cache
+    (key-range split, packed rows), decode-sized calls (m * group_size <= 16), and ragged cases where the
+    cache length cuts the rows.  Rows past n are poisoned."""
+    import random
+    ops = _ops()
+    rnd = random.Random(20251125)
+    for it in range(48):
+        Hkv = rnd.choice([1, 2, 3, 4, 8])
+        g = rnd.choice([1, 1, 2, 5, 6, 7, 16])
+        H = Hkv * g
+        kind = ("square", "chunk", "decode", "ragged")[it % 4]
+        if kind == "square":
+            m = rnd.randint(1, 700)
+            n, off = m, 0
+        elif kind == "chunk":
+            m = rnd.randint(1, 130)
+            n = rnd.randint(2048, 9000)
+            off = n - m
+        elif kind == "decode":
+            m = rnd.randint(1, max(1, 16 // g))
+            n = rnd.randint(1, 6000)
+            off = max(0, n - m)
+        else:
+            m = rnd.randint(1, 300)
+            off = rnd.randint(0, 500)
+            n = rnd.randint(1, m + off + 50)
+        dt = DT_BFLOAT16 if rnd.random() < 0.5 else DT_FLOAT16
+        q = normal_bits(17000 + it, (m, H, 128), dt)
+        k = normal_bits(18000 + it, (n + 3, Hkv, 128), dt)
+        v = normal_bits(19000 + it, (n + 3, Hkv, 128), dt)
+        k[n:] = 0x7FFF
+        v[n:] = 0x7FFF
+        d_out = dev_empty(q.shape)
+        print(f"case {it}: {kind} m={m} n={n} offset={off} H={H} Hkv={Hkv} dt={dt}", flush=True)
+        ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), m, n, off, g, Hkv, 128, dt)
+        check_attention(to_host(d_out), q, k, v, n, off, dt)
+
+
 @pytest.mark.parametrize("dt", [DT_FLOAT16, DT_BFLOAT16])
 @pytest.mark.parametrize("is_neox", [False, True])
 @pytest.mark.parametrize("H,Hkv", [(12, 2), (32, 32), (40, 8), (28, 4)])

@@ -105,11 +105,16 @@ def test_default_workspace_size_covers_the_default_split_count():
     """num_splits <= 0 sizes the workspace for the largest count the default rule can pick, so a
     caller that lets the decode call choose never gets LLMHIP_ERR_WORKSPACE."""
     import llm_simple_amd.ops as ops
-    for batch, hkv in ((1, 8), (16, 8), (3, 2), (1, 1), (64, 8)):
+    for batch, hkv in ((1, 8), (16, 8), (3, 2), (1, 1), (64, 8), (20, 8), (24, 8), (40, 8), (48, 8), (12, 8), (7, 3)):
         cover = ops.flash_decode_workspace_bytes(batch, 5, hkv, 128, 0)
-        for n in (1, 100, 4096, 32768, 131072):
+        for n in (1, 100, 129, 4096, 8192, 32768, 131072):
             s = ops.flash_decode_default_splits(batch, n, hkv)
+            assert 1 <= s <= max(1, -(-n // 128)), (batch, hkv, n, s)  # every split holds at least one block
             assert ops.flash_decode_workspace_bytes(batch, 5, hkv, 128, s) <= cover, (batch, hkv, n)
+    # the rule fills whole rounds of 256 workgroups where the pair count does not divide one
+    assert ops.flash_decode_default_splits(40, 8192, 8) == 4    # 320 pairs -> 1280 workgroups = 5 rounds
+    assert ops.flash_decode_default_splits(24, 8192, 8) == 4    # 192 pairs -> 768 = 3 rounds
+    assert ops.flash_decode_default_splits(64, 4096, 8) == 1    # 512 pairs = 2 rounds already
 
 
 def test_sanitizer_builds_of_oracle_and_device_layer():

@@ -552,8 +552,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
       const int key0 = j * kTileN + kw0;
       if ((key0 + kWaveKeys - 1 > tok_lo + offset_) || (key0 + kWaveKeys > n_))
         w.mask(s_cur, key0, qtok, offset_, n_);
-      // a burst of loads would stall every wave behind the texture addresser's queue:
-      // one load every 8 * KB / PER MFMAs instead
+      // In the 8-wave kernel a burst of loads would stall every wave behind the texture addresser's
+      // queue: one load every 8 * KB / PER MFMAs instead.  The 4-wave kernels run where a step is
+      // short against a memory round trip, and issue a phase's loads beside its first MFMAs
+      // (S=2560: 61.0 -> 59.1 us, S=3072: 76.3 -> 75.0 us; the 8-wave kernel loses 0.7 % that way).
       // (Paired waves, KB == 1, run short sequences, where a step is shorter than a memory round
       // trip: there all loads of a step go out with its first MFMAs.)
       auto k_hook = [&](int i) {
@@ -562,7 +564,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
           if (KB == 1) {
             if (i == r) ld.template issue<false>(kbase, jk, kslot * kTileBytes, r);
             if (i == PER + r) ld.template issue<true>(vbase, jv, kVRegion + vslot * kTileBytes, r);
-          } else if (i == (8 * KB / PER) * r + 1) {
+          } else if (i == (NW == 4 ? r : (8 * KB / PER) * r + 1)) {
             ld.template issue<false>(kbase, jk, kslot * kTileBytes, r);
           }
         }
@@ -579,7 +581,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
       w.pv(lds, slot * kTileBytes, [&](int i) {
 #pragma unroll
         for (int r = 0; r < PER; ++r)
-          if (KB != 1 && i == (8 * KB / PER) * r + 1)
+          if (KB != 1 && i == (NW == 4 ? r : (8 * KB / PER) * r + 1))
             ld.template issue<true>(vbase, jv, kVRegion + vslot * kTileBytes, r);
       });
     } else {

@@ -639,19 +639,40 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(PrefillParams p) {
   const size_t slot = (size_t)blockIdx.x * 8 + (threadIdx.x >> 5);
   const int d4 = threadIdx.x & 31;
   if (slot >= stride) return;
-  float M = -INFINITY;
-  for (int s = 0; s < p.num_splits; ++s) M = fmaxf(M, p.ws_ml[(s * stride + slot) * 2]);
-  const float M_use = (M == -INFINITY) ? 0.0f : M;
-  float L = 0.0f;
+  // One pass, four key ranges per round: all loads of a round are issued before any is used, and the
+  // running reference maximum moves between rounds (a pass for the maximum first would be one memory
+  // round trip per key range).
+  const int S = p.num_splits;
+  float M = -INFINITY, L = 0.0f;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-  for (int s = 0; s < p.num_splits; ++s) {
-    const float *ml = p.ws_ml + (s * stride + slot) * 2;
-    const float wt = fast_exp2((ml[0] - M_use) * p.scale_log2e);  // exp2(-inf) = 0 for an empty range
-    L += wt * ml[1];
-    const f32x4_t o = *reinterpret_cast<const f32x4_t *>(p.ws_o + (s * stride + slot) * kHeadDim + 4 * d4);
+  for (int s0 = 0; s0 < S; s0 += 4) {
+    float mv[4], lv[4];
+    f32x4_t ov[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[i] += wt * o[i];
+    for (int j = 0; j < 4; ++j) {
+      const size_t at = (size_t)min(s0 + j, S - 1) * stride + slot;
+      mv[j] = p.ws_ml[at * 2];
+      lv[j] = p.ws_ml[at * 2 + 1];
+      ov[j] = *reinterpret_cast<const f32x4_t *>(p.ws_o + at * kHeadDim + 4 * d4);
+    }
+    float Mn = M;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (s0 + j < S) Mn = fmaxf(Mn, mv[j]);
+    const float M_use = (Mn == -INFINITY) ? 0.0f : Mn;
+    const float resc = fast_exp2((M - M_use) * p.scale_log2e);  // 0 on the first round (M = -inf)
+    L *= resc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] *= resc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      // exp2(-inf) = 0 for an empty range
+      const float wt = (s0 + j < S) ? fast_exp2((mv[j] - M_use) * p.scale_log2e) : 0.0f;
+      L += wt * lv[j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] += wt * ov[j][i];
+    }
+    M = Mn;
   }
   const float inv = (L > 0.0f) ? 1.0f / L : 0.0f;
   u32x2_t w;

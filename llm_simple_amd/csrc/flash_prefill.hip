@@ -681,6 +681,76 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(PrefillParams p) {
   *reinterpret_cast<u32x2_t *>(p.out + slot * kRowBytes + d4 * 8) = w;
 }
 
+// The same fold for few output rows and many key ranges (a short chunk over a very long cache): one
+// (row, head) slot per workgroup, its key ranges dealt to 8 groups of 32 threads (group sg takes ranges
+// sg, sg + 8, ..., four per round), the groups merged through LDS -- the slots alone would not fill
+// the chip and every thread would walk all ranges.  grid = m * H.
+template <typename T>
+__global__ __launch_bounds__(256) void prefill_combine_wide_kernel(PrefillParams p) {
+  using E = Elem<T>;
+  __shared__ float red_m[8], red_l[8];
+  __shared__ f32x4_t red_o[8][32];
+  const size_t stride = (size_t)p.m * p.H, slot = blockIdx.x;
+  const int sg = threadIdx.x >> 5, d4 = threadIdx.x & 31;
+  const int S = p.num_splits;
+  float M = -INFINITY, L = 0.0f;
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = sg; s0 < S; s0 += 32) {
+    float mv[4], lv[4];
+    f32x4_t ov[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const size_t at = (size_t)min(s0 + 8 * j, S - 1) * stride + slot;
+      mv[j] = p.ws_ml[at * 2];
+      lv[j] = p.ws_ml[at * 2 + 1];
+      ov[j] = *reinterpret_cast<const f32x4_t *>(p.ws_o + at * kHeadDim + 4 * d4);
+    }
+    float Mn = M;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (s0 + 8 * j < S) Mn = fmaxf(Mn, mv[j]);
+    const float M_use = (Mn == -INFINITY) ? 0.0f : Mn;
+    const float resc = fast_exp2((M - M_use) * p.scale_log2e);
+    L *= resc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] *= resc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float wt = (s0 + 8 * j < S) ? fast_exp2((mv[j] - M_use) * p.scale_log2e) : 0.0f;
+      L += wt * lv[j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] += wt * ov[j][i];
+    }
+    M = Mn;
+  }
+  if (d4 == 0) {
+    red_m[sg] = M;
+    red_l[sg] = L;
+  }
+  red_o[sg][d4] = acc;
+  __syncthreads();
+  if (sg != 0) return;
+  float Mt = -INFINITY;
+#pragma unroll
+  for (int g8 = 0; g8 < 8; ++g8) Mt = fmaxf(Mt, red_m[g8]);
+  const float Mt_use = (Mt == -INFINITY) ? 0.0f : Mt;
+  float Lt = 0.0f;
+  f32x4_t tot = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int g8 = 0; g8 < 8; ++g8) {
+    const float wt = fast_exp2((red_m[g8] - Mt_use) * p.scale_log2e);  // 0 for a group without ranges (-inf)
+    Lt += wt * red_l[g8];
+    const f32x4_t o = red_o[g8][d4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) tot[i] += wt * o[i];
+  }
+  const float inv = (Lt > 0.0f) ? 1.0f / Lt : 0.0f;
+  u32x2_t w;
+  w[0] = E::pack2(tot[0] * inv, tot[1] * inv);
+  w[1] = E::pack2(tot[2] * inv, tot[3] * inv);
+  *reinterpret_cast<u32x2_t *>(p.out + slot * kRowBytes + d4 * 8) = w;
+}
+
 template <typename T, int NW, int KB = 2>
 static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) {
   PrefillParams p = p0;
@@ -726,7 +796,11 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
   hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds_bytes, stream, p);
   e = hipGetLastError();
   if (e != hipSuccess || p.num_splits == 1) return e;
-  hipLaunchKernelGGL(prefill_combine_kernel<T>, dim3((unsigned)(((size_t)p.m * p.H + 7) / 8)), dim3(256), 0, stream, p);
+  const size_t slots = (size_t)p.m * p.H;
+  if (slots <= 2048 && p.num_splits >= 8)
+    hipLaunchKernelGGL(prefill_combine_wide_kernel<T>, dim3((unsigned)slots), dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL(prefill_combine_kernel<T>, dim3((unsigned)((slots + 7) / 8)), dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -409,7 +409,7 @@ __device__ __forceinline__ void store_partial(const WaveAttn<T, KB> &w, float *o
 // so a load costs no vector ALU work.  The loads are issued from inline asm: the compiler
 // would order every later LDS read behind a transfer it knows about (s_waitcnt vmcnt(0)).
 // Completion is waited for explicitly before the barrier that publishes a stage.
-template <int NW> struct DirectLoader {
+template <int NW, bool NT> struct DirectLoader {
   static constexpr int kSlots = 16 / NW;  // instructions per wave per tile
   int n, row_bytes;
   uint32_t lds_row0;          // LDS byte offset of row 4*wave (wave-uniform)
@@ -430,11 +430,20 @@ template <int NW> struct DirectLoader {
       asm volatile("" : "+v"(row[s]), "+v"(lane_k[s]), "+v"(lane_v[s]));
     }
   }
+  // NT: the tile is read by this workgroup only (a packed chunk of one tile per kv head over a long
+  // cache): non-temporal, like the decode kernel's loads (4 tokens over 131072 keys: 106 -> 93 us);
+  // tiles that several workgroups read stay ordinary loads (non-temporal costs those 3-10 %).
   static __device__ __forceinline__ void dma(const char *tile_base, uint32_t lane_off, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(lane_off), "s"(tile_base), "s"(lds_addr)
-                 : "m0");
+    if (NT)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                   :
+                   : "v"(lane_off), "s"(tile_base), "s"(lds_addr)
+                   : "m0");
+    else
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(lane_off), "s"(tile_base), "s"(lds_addr)
+                   : "m0");
   }
   // t: key tile; lds_tile: LDS byte offset of the destination tile
   template <bool IS_V>
@@ -460,7 +469,7 @@ template <int NW> struct DirectLoader {
 // about one 128-row workgroup per CU, where the serial MFMA chain of a wave is what the launch
 // waits for.
 // ---------------------------------------------------------------------------
-template <typename T, int NW, int KB>
+template <typename T, int NW, int KB, bool NT>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel(PrefillParams p) {
   // SUB tiles of 64 keys per stage and per barrier: with one workgroup per CU (NW = 8) a stage
   // holds 128 keys, which halves the number of times the waves are forced in step.
@@ -527,7 +536,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   }
   w.load_q(p.q + (size_t)qtok * q_row_bytes + (size_t)qhead * kRowBytes);
 
-  DirectLoader<NW> ld;
+  DirectLoader<NW, NT> ld;
   ld.init(wave, lane, kv_row_bytes, n_);
   // K runs one tile ahead of V: S(j+1) = K(j+1) Q^T is issued together with the softmax of
   // tile j, so K tile t is fetched SUB+1 iterations and V tile t SUB iterations before use.
@@ -780,9 +789,13 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
     grid = T_ * p.H * S_;
   }
   const size_t lds_bytes = (NW == 8 ? 2 : 1) * 4 * kTileBytes;
-  void (*kern)(PrefillParams) = flash_prefill_kernel<T, NW, KB>;
+  // packed rows, one tile per kv head: every K/V tile is read by one workgroup only (KB == 2 there)
+  const bool nt = KB == 2 && p.pack && T_ == 1;
+  void (*kern)(PrefillParams) = flash_prefill_kernel<T, NW, KB, false>;
+  if (nt) kern = flash_prefill_kernel<T, NW, KB, (KB == 2)>;
   // the opt-in for more than 64 KiB of dynamic LDS is per device: once per device and kernel
-  static std::atomic<uint64_t> attr_done{0};
+  static std::atomic<uint64_t> attr_done_both[2];
+  std::atomic<uint64_t> &attr_done = attr_done_both[nt ? 1 : 0];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;

@@ -429,6 +429,24 @@ def test_long_context_131072():
         check_attention(to_host(d_out), q, k, v, n, n - m, dt)
 
 
+@pytest.mark.parametrize("dt", [DT_BFLOAT16, DT_FLOAT16])
+def test_short_chunk_over_131072_keys_two_kv_heads(dt):
+    """The Qwen2.5-1.5B head counts (12 query heads on 2 kv heads): 9 new tokens over a 131072-key cache run
+    as 54 packed rows per kv head over 128 key ranges, each K/V tile read by one workgroup (non-temporal
+    loads), folded by the combine kernel for few rows and many ranges."""
+    ops = _ops()
+    H, Hkv, n, m = 12, 2, 131072, 9
+    q = normal_bits(1410, (m, H, 128), dt)
+    k = normal_bits(1411, (n + 2, Hkv, 128), dt)
+    v = normal_bits(1412, (n + 2, Hkv, 128), dt)
+    k[n:] = 0x7FFF
+    v[n:] = 0x7FFF
+    assert ops.lib.llmhip_flash_attn_scratch_bytes(m, n, n - m, H // Hkv, Hkv) == 128 * m * H * 130 * 4
+    d_out = dev_empty(q.shape)
+    ops.hip_flash_attn_gqa_layer(d_out, to_dev(q), to_dev(k), to_dev(v), m, n, n - m, H // Hkv, Hkv, 128, dt)
+    check_attention(to_host(d_out), q, k, v, n, n - m, dt)
+
+
 def test_flash_decode_random_shapes():
     """Seeded sweep of the batched decode entry point: batch, KV length, allocated rows per sequence, group
     size and kv heads drawn at random (group sizes up to the 16 columns of the kernel), default splits."""

@@ -45,8 +45,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("decode", 16, 32768): (2097637 + 656) * 1024,         # algorithmic 2097152 KiB
     ("decode", 1, 32768): (131317 + 656) * 1024,           # algorithmic 131072 KiB
     ("rope", 4096): (40753 + 36864) * 1024,                # algorithmic 75776 KiB
-    ("chunked", 256, 33024): (136014 + 33557 + 33339 + 1792) * 1024,   # prefill kernel + combine
-    ("chunked", 40, 131072): (524998 + 26241 + 26437 + 400) * 1024,
+    ("chunked", 256, 33024): (136014 + 33556 + 33282 + 1792) * 1024,   # prefill kernel + combine
+    ("chunked", 40, 131072): (537483 + 26242 + 28843 + 400) * 1024,
 }
 
 

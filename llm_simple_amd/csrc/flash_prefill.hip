@@ -19,12 +19,14 @@
 // moves lazily, so O is rarely rescaled.  Accumulation is fp32; out =
 // O / l rounded once; l sums the ROUNDED probabilities (what P.V used).
 //
-// flash_prefill_kernel<T, NW, KB>: NW waves share the K/V tiles of 16*NW*KB query rows.
+// flash_prefill_kernel<T, NW, KB, NT>: NW waves share the K/V tiles of 16*NW*KB query rows.
 // NW = 8, KB = 2 (256 rows, one workgroup per CU) once there are about 1.5 such workgroups per CU;
 // NW = 4, KB = 2 (128 rows, two workgroups per CU) below that; NW = 8, KB = 1 (128 rows, two waves
-// per row block, each taking one 32-key half of every tile) up to two 128-row workgroups per CU.
+// per row block, each taking one 32-key half of every tile) up to two 128-row workgroups per CU;
+// NW = 4, KB = 1 (64 rows, paired waves, two workgroups per CU) up to about 1.2 per CU.  NT: the
+// tile loads are non-temporal (chunks whose K/V tiles only one workgroup reads).
 // Tiles travel global -> LDS without VGPR staging (global_load_lds_dwordx4), spread over the MFMA
-// stream.  The loop is software pipelined inside a wave: the MFMAs of S(j+1) are issued beside the
+// stream in the 8-wave kernels, issued beside the first MFMAs of a phase in the 4-wave ones.  The loop is software pipelined inside a wave: the MFMAs of S(j+1) are issued beside the
 // softmax of tile j (the first ones beside the row-maximum chain, the rest, together with the
 // MFMAs of P(j).V(j), beside the exponentials), so K is fetched one tile ahead of V.
 // Every LDS fragment address is a loop-invariant register plus an immediate, and a
@@ -33,8 +35,8 @@
 //
 // A chunk of few query rows over a long cache (chunked prefill) has its key range split over
 // workgroups: each leaves an fp32 partial (reference maximum, sum, unnormalised O) and
-// prefill_combine_kernel folds them; a chunk shorter than a tile packs the query heads of a kv
-// head into the rows of one tile.  plan_prefill decides all of this from the shape and the
+// prefill_combine_kernel (or, for few rows and many ranges, prefill_combine_wide_kernel) folds
+// them; a chunk shorter than a tile packs the query heads of a kv head into the rows of one tile.  plan_prefill decides all of this from the shape and the
 // device's CU count.
 #include <atomic>
 

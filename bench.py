@@ -122,7 +122,7 @@ def torch_int16():
     return torch.int16
 
 
-def bench_prefill(ops, torch, timer, S, steps, warmup, H=28, Hkv=4, clock=False):
+def bench_prefill(ops, torch, timer, S, steps, warmup, H=28, Hkv=4, clock=False, bops=None):
     g = torch.Generator(device="cuda").manual_seed(1004 + S)
     q = torch.randn(S, H, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
     k = torch.randn(S, Hkv, 128, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
@@ -144,7 +144,7 @@ def bench_prefill(ops, torch, timer, S, steps, warmup, H=28, Hkv=4, clock=False)
         probe = torch.zeros(2, dtype=torch.int64, device="cuda")
         for _ in range(20):
             step(0)
-        ops.hip_flash_attn_gqa_clocked_layer(out, q, k, v, S, S, 0, H // Hkv, Hkv, 128, DT_BF16, probe)
+        bops.hip_flash_attn_gqa_clocked_layer(out, q, k, v, S, S, 0, H // Hkv, Hkv, 128, DT_BF16, probe)
         torch.cuda.synchronize()
         ticks, ref = (int(x) for x in probe.cpu())
         if ref > 0:
@@ -192,7 +192,7 @@ def bench_chunked_prefill(ops, torch, timer, m, n, steps, warmup, H=28, Hkv=4):
             "kv_gbs": 2.0 * n * Hkv * 256 / (ev_ms * 1e-3) / 1e9, "max_abs_err": worst}
 
 
-def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
+def bench_decode(ops, bops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
     """Cold numbers: successive launches walk over distinct KV buffers whose total
     exceeds 1 GiB, so no launch is served from the 256 MB last-level cache."""
     kv_bytes = 2 * batch * n * Hkv * 128 * 2
@@ -223,8 +223,8 @@ def bench_decode(ops, torch, timer, batch, n, steps, warmup, H=40, Hkv=8):
     hot_ms, _, _ = timed(torch, timer, hot, reps)
     # a kernel that only reads the same K and V arrays, cold like `step`: what the memory system delivers at
     # this byte count (the better of its two launch shapes)
-    sink = torch.empty(ops.STREAM_READ_SINK_BYTES, dtype=torch.uint8, device="cuda")
-    read_ms = min(timed(torch, timer, lambda i, var=var: ops.probe_stream_read(ks[i % nbuf], vs[i % nbuf], sink, var),
+    sink = torch.empty(bops.STREAM_READ_SINK_BYTES, dtype=torch.uint8, device="cuda")
+    read_ms = min(timed(torch, timer, lambda i, var=var: bops.probe_stream_read(ks[i % nbuf], vs[i % nbuf], sink, var),
                         reps)[0] for var in (0, 1))
     torch.cuda.synchronize()
     # accuracy of the last timed (hot) launch: sequence 0 and the last one against the fp32 oracle
@@ -429,6 +429,7 @@ def main():
 
     import torch
     import llm_simple_amd.ops as ops
+    import llm_simple_amd.bench_ops as bops  # the measurement library: clock stamp, MFMA ceiling, plain read
     if not torch.cuda.is_available():
         log("bench.py: no GPU visible")
         sys.exit(1)
@@ -446,8 +447,8 @@ def main():
     # instructions of an attention inner loop beside the MFMAs (no memory traffic, no barriers)
     ceiling = None
     if "ceiling" in legs:
-        ceiling = {"mfma_only_tflops": ops.probe_mfma_ceiling(0, 150.0),
-                   "attention_mix_tflops": ops.probe_mfma_ceiling(1, 150.0),
+        ceiling = {"mfma_only_tflops": bops.probe_mfma_ceiling(0, 150.0),
+                   "attention_mix_tflops": bops.probe_mfma_ceiling(1, 150.0),
                    "what": "sustained bf16 32x32x16 MFMA rate on N(0,1) operands, 8 waves per CU: the MFMAs alone, "
                            "and with 6 LDS fragment reads, 13 vector instructions and 4 v_exp_f32 per 4 MFMAs "
                            "beside them (the prefill loop's mix) -- no memory traffic, barriers or dependences"}
@@ -456,7 +457,7 @@ def main():
 
     # ---- the timed step: prefill at the headline shape ----
     torch.cuda.synchronize()
-    pre, _ = bench_prefill(ops, torch, timer, args.seq, args.steps, args.warmup, clock=True)
+    pre, _ = bench_prefill(ops, torch, timer, args.seq, args.steps, args.warmup, clock=True, bops=bops)
     log(f"prefill S={args.seq}: {pre['ms_event'] * 1e3:.1f} us  {pre['tflops']:.1f} TFLOP/s  "
         f"max-abs {pre['max_abs_err']:.2e}  shader clock {pre.get('shader_clock_mhz', 0):.0f} MHz")
     if "prefill" in legs:
@@ -483,7 +484,7 @@ def main():
         dec = []
         shapes = [tuple(int(x) for x in c.split("x")) for c in args.decode_shapes.split(",") if c]
         for batch, n in shapes:
-            r = bench_decode(ops, torch, timer, batch, n, args.steps, args.warmup)
+            r = bench_decode(ops, bops, torch, timer, batch, n, args.steps, args.warmup)
             log(f"decode B={batch} n={n} splits={r['splits']}: cold {r['ms_cold'] * 1e3:.1f} us "
                 f"{r['gbs_cold']:.0f} GB/s, hot {r['ms_hot'] * 1e3:.1f} us {r['gbs_hot']:.0f} GB/s, "
                 f"max-abs {r['max_abs_err']:.2e}; a plain read of the same arrays, cold: "
@@ -501,7 +502,7 @@ def main():
             "box": {"plain_read_gbs": head["gbs_plain_read"],
                     "frac_of_plain_read": head["gbs_cold"] / head["gbs_plain_read"],
                     "plain_read": "a kernel that only reads the same K and V arrays once, cold, timed the same way "
-                                  "(llmhip_probe_stream_read)"},
+                                  "(llmhip_bench_stream_read)"},
             "workload": f"Qwen2.5-32B decode bf16 H=40 Hkv=8 n={head['n']} batch={head['batch']} "
                         f"({head['kv_bytes'] / 2 ** 20:.0f} MiB of K+V per launch, cold)"}
         extra["decode_all"] = [

@@ -75,16 +75,6 @@ int llmhip_flash_attn_opt_prefill(void *out, const void *q, const void *k, const
  * stream up with its largest shape. */
 size_t llmhip_flash_attn_scratch_bytes(int m, int n, int offset, int group_size, int kv_head_num);
 
-/* Measurement aid with no counterpart in the reference: llmhip_flash_attn_gqa on the prefill
- * kernel (m * group_size > 16, LLMHIP_ERR_UNSUPPORTED otherwise) that also makes the first
- * scheduled workgroup store two 64-bit counters at clock_probe (device memory, 16 bytes): the
- * shader-clock ticks and the ticks of the constant 100 MHz reference clock between its start
- * and its end.  Their ratio x 100 MHz is the shader clock under this kernel's load, which the
- * benchmark prints next to the peak it prices against. */
-int llmhip_flash_attn_gqa_clocked(void *out, const void *q, const void *k, const void *v, int m,
-                                  int n, int offset, int group_size, int kv_head_num, int head_dim,
-                                  int dt, void *clock_probe, void *stream);
-
 /* Batched split-KV decode over a contiguous per-sequence KV cache: one query
  * token per sequence, `batch` independent sequences of the same valid length n.
  * q, out: [batch][group_size*kv_head_num][head_dim];
@@ -186,26 +176,9 @@ int llmhip_rope_kv_append(void *out_q, void *k_cache, void *v_cache, const void 
  * aclrtSynchronizeStream (src/llama2_layer_npu.cpp:605-608) and the event
  * calls of src/profiling.cpp:48-78. */
 int llmhip_device_count(void);
-/* Compute units, maximum shader clock (kHz) and memory size of a device (any pointer may be null);
- * what the benchmark derives the box's own peak from. */
+/* Compute units, maximum shader clock (kHz) and memory size of a device (any pointer may be null):
+ * hipGetDeviceProperties for host code that includes no HIP header. */
 int llmhip_device_props(int device, int *compute_units, int *max_clock_khz, size_t *total_mem_bytes);
-/* Measurement aid with no counterpart in the reference: runs, for about target_ms (<= 2000), a loop of
- * back-to-back bf16 32x32x16 MFMAs on N(0,1) operands on every CU and returns the sustained TFLOP/s.
- * mix 0: the MFMAs alone (what the matrix pipe sustains at the clock its own power draw allows);
- * mix 1: the same MFMAs with the LDS fragment reads and vector instructions of a flash-attention
- * inner loop beside them, no memory traffic, no barriers, no dependences: an upper bound for any
- * attention kernel with that instruction mix on this machine.  The benchmark prints both next to
- * the published peak.  Allocates and frees two small device buffers; runs on the default stream. */
-int llmhip_probe_mfma_ceiling(int mix, double target_ms, double *tflops);
-/* Measurement aid, no counterpart in the reference: a plain streaming read of two device arrays of
- * bytes_each bytes (a multiple of 16), every byte read once and nothing else done -- what the memory
- * system delivers to a kernel that only reads, to set beside the decode kernel's rate on the same byte
- * count.  variant 0: one workgroup per CU with 8 loads in flight per thread; variant 1: two per CU with
- * 4 (the better one below about 256 MiB).  sink: LLMHIP_STREAM_READ_SINK_BYTES bytes of device memory
- * that receive a checksum per wave.  Asynchronous on `stream`; allocates nothing. */
-#define LLMHIP_STREAM_READ_SINK_BYTES 65536
-int llmhip_probe_stream_read(const void *src_a, const void *src_b, size_t bytes_each, void *sink,
-                             size_t sink_bytes, int variant, void *stream);
 int llmhip_set_device(int device);
 int llmhip_malloc(void **ptr, size_t bytes);
 int llmhip_free(void *ptr);

@@ -17,10 +17,10 @@
 
 #include <vector>
 
+#include "bench_kernels.hpp"
 #include "common.hpp"
-#include "kernels.hpp"
 
-namespace llmhip {
+namespace LLMHIP_NS {
 
 namespace {
 
@@ -197,4 +197,4 @@ hipError_t run_mfma_ceiling(int mix, double target_ms, double *tflops_out) {
   return e == hipSuccess ? hipGetLastError() : e;
 }
 
-}  // namespace llmhip
+}  // namespace LLMHIP_NS

@@ -14,7 +14,16 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-namespace llmhip {
+// The measurement library (libllmhip_bench.so) compiles the prefill kernel a second time with
+// LLMHIP_BENCH defined (a clock stamp in the kernel); its copy lives in a namespace of its own so
+// that the two libraries never share a symbol.
+#ifdef LLMHIP_BENCH
+#define LLMHIP_NS llmhip_bench
+#else
+#define LLMHIP_NS llmhip
+#endif
+
+namespace LLMHIP_NS {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
@@ -158,4 +167,4 @@ __device__ __forceinline__ u32x4_t global_load_b128_nt(const void *p) {
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
 }
 
-}  // namespace llmhip
+}  // namespace LLMHIP_NS

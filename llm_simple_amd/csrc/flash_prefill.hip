@@ -43,7 +43,7 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
-namespace llmhip {
+namespace LLMHIP_NS {
 
 constexpr int kTileN = 64;                      // keys per LDS tile
 constexpr int kTileBytes = kTileN * kRowBytes;  // 16 KiB
@@ -71,8 +71,10 @@ struct PrefillParams {
   int pack;
   float *ws_o;            // [split][m][H][128]
   float *ws_ml;           // [split][m][H][2]
-  // measurement aid, normally null: workgroup 0 stores {shader-clock ticks, 100 MHz ticks} of its lifetime
+#ifdef LLMHIP_BENCH
+  // measurement library only: workgroup 0 stores {shader-clock ticks, 100 MHz ticks} of its lifetime
   unsigned long long *clock_probe;
+#endif
 };
 
 // blockIdx -> (query tile, head, key range).  Workgroup ids are dealt round-robin to the 8
@@ -485,11 +487,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tile, head, split;
   if (!prefill_schedule(p, blockIdx.x, tile, head, split)) return;
+#ifdef LLMHIP_BENCH
   unsigned long long clk0 = 0, ref0 = 0;
   if (p.clock_probe) {
     clk0 = __builtin_amdgcn_s_memtime();
     ref0 = __builtin_amdgcn_s_memrealtime();
   }
+#endif
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int kvh = head / p.g;
@@ -635,10 +639,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flash_prefill_kernel
   else
     w.store(lds + rb * 32 * kRowBytes, p.out + (size_t)qblk0 * q_row_bytes + (size_t)head * kRowBytes,
             q_row_bytes, p.m - qblk0);
+#ifdef LLMHIP_BENCH
   if (p.clock_probe && blockIdx.x == 0 && tid == 0) {
     p.clock_probe[0] = __builtin_amdgcn_s_memtime() - clk0;
     p.clock_probe[1] = __builtin_amdgcn_s_memrealtime() - ref0;
   }
+#endif
 }
 
 // Folds the key-range partials of the output rows with the log-sum-exp rule.  256 threads handle 8
@@ -906,11 +912,18 @@ size_t flash_prefill_workspace_bytes(int m, int n, int offset, int group_size, i
   return (size_t)pl.num_splits * m * H * (kHeadDim + 2) * sizeof(float);
 }
 
+#ifdef LLMHIP_BENCH
 hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
                                 int n, int offset, int group_size, int kv_head_num, int dt,
                                 hipStream_t stream, void *workspace, void *clock_probe) {
   PrefillParams p;
   p.clock_probe = static_cast<unsigned long long *>(clock_probe);
+#else
+hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
+                                int n, int offset, int group_size, int kv_head_num, int dt,
+                                hipStream_t stream, void *workspace) {
+  PrefillParams p;
+#endif
   p.q = static_cast<const char *>(q);
   p.k = static_cast<const char *>(k);
   p.v = static_cast<const char *>(v);
@@ -943,4 +956,4 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
   return f16 ? launch_prefill_t<_Float16, 4>(p, stream) : launch_prefill_t<__bf16, 4>(p, stream);
 }
 
-}  // namespace llmhip
+}  // namespace LLMHIP_NS

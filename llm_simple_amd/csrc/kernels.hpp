@@ -5,16 +5,24 @@
 #include <stddef.h>
 #include <stdint.h>
 
-namespace llmhip {
+#include "common.hpp"
+
+namespace LLMHIP_NS {
 
 // workspace: device memory of flash_prefill_workspace_bytes() bytes (0 = none needed) for the fp32
 // partials of a key-range split; with a null workspace the call runs unsplit.
-// clock_probe: null, or a device pointer to two 64-bit counters that workgroup 0 fills with the
-// shader-clock ticks and the reference-clock ticks of its lifetime (measurement aid).
 size_t flash_prefill_workspace_bytes(int m, int n, int offset, int group_size, int kv_head_num);
+#ifdef LLMHIP_BENCH
+// The measurement library's copy: clock_probe is a device pointer to two 64-bit counters that
+// workgroup 0 fills with the shader-clock ticks and the reference-clock ticks of its lifetime.
 hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
                                 int n, int offset, int group_size, int kv_head_num, int dt,
-                                hipStream_t stream, void *workspace = nullptr, void *clock_probe = nullptr);
+                                hipStream_t stream, void *workspace, void *clock_probe);
+#else
+hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const void *v, int m,
+                                int n, int offset, int group_size, int kv_head_num, int dt,
+                                hipStream_t stream, void *workspace = nullptr);
+#endif
 
 // Split-KV decode.  rows = m * group_size <= 16 query rows per kv head.
 size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,
@@ -56,11 +64,4 @@ void release_matmul_resources();
 hipError_t launch_add(void *out, const void *lhs, const void *rhs, size_t total, int dt,
                       hipStream_t stream);
 
-// Measurement aid (ceiling_probe.hip): sustained MFMA TFLOP/s of this GPU on N(0,1) bf16 operands,
-// mix 0 = MFMAs alone, mix 1 = MFMAs with the LDS reads and vector instructions of an attention loop.
-hipError_t run_mfma_ceiling(int mix, double target_ms, double *tflops_out);
-hipError_t launch_stream_read(const void *a, const void *b, size_t bytes_each, void *sink, int variant,
-                              hipStream_t stream);
-constexpr size_t kStreamReadSinkBytes = 65536;  // 4 bytes per wave of the largest grid (2 workgroups per CU)
-
-}  // namespace llmhip
+}  // namespace LLMHIP_NS

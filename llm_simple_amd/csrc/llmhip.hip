@@ -116,21 +116,6 @@ int llmhip_flash_attn_opt_prefill(void *out, const void *q, const void *k, const
   return attn_common(out, q, k, v, m, n, offset, 1, head_num, head_dim, dt, stream);
 }
 
-int llmhip_flash_attn_gqa_clocked(void *out, const void *q, const void *k, const void *v, int m,
-                                  int n, int offset, int group_size, int kv_head_num, int head_dim,
-                                  int dt, void *clock_probe, void *stream) {
-  if (!out || !q || !k || !v || !clock_probe || !all_aligned16(out, q, k, v) ||
-      (reinterpret_cast<uintptr_t>(clock_probe) & 7u))
-    return LLMHIP_ERR_INVALID_ARG;
-  if (m < 1 || n < 1 || offset < 0 || group_size < 1 || kv_head_num < 1 || !dtype_ok(dt))
-    return LLMHIP_ERR_INVALID_ARG;
-  if (head_dim != 128) return LLMHIP_ERR_UNSUPPORTED;
-  if (kv_head_num > 65535 || (long long)group_size * kv_head_num > 65535) return LLMHIP_ERR_UNSUPPORTED;
-  if ((long long)m * group_size <= kMaxDecodeCols) return LLMHIP_ERR_UNSUPPORTED;  // prefill kernel only
-  return from_hip(launch_flash_prefill(out, q, k, v, m, n, offset, group_size, kv_head_num, dt,
-                                       as_stream(stream), nullptr, clock_probe));
-}
-
 size_t llmhip_flash_attn_scratch_bytes(int m, int n, int offset, int group_size, int kv_head_num) {
   if (m < 1 || n < 1 || offset < 0 || group_size < 1 || kv_head_num < 1) return 0;
   if ((long long)m * group_size <= kMaxDecodeCols) {
@@ -285,20 +270,6 @@ int llmhip_device_props(int device, int *compute_units, int *max_clock_khz, size
   if (max_clock_khz) *max_clock_khz = prop.clockRate;
   if (total_mem_bytes) *total_mem_bytes = prop.totalGlobalMem;
   return LLMHIP_OK;
-}
-int llmhip_probe_mfma_ceiling(int mix, double target_ms, double *tflops) {
-  if (!tflops || (mix != 0 && mix != 1) || target_ms < 0.0 || target_ms > 2000.0) return LLMHIP_ERR_INVALID_ARG;
-  if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;
-  return from_hip(run_mfma_ceiling(mix, target_ms, tflops));
-}
-int llmhip_probe_stream_read(const void *src_a, const void *src_b, size_t bytes_each, void *sink, size_t sink_bytes,
-                             int variant, void *stream) {
-  if (!src_a || !src_b || !sink || bytes_each == 0 || bytes_each % 16 != 0 || (variant != 0 && variant != 1))
-    return LLMHIP_ERR_INVALID_ARG;
-  if (sink_bytes < kStreamReadSinkBytes) return LLMHIP_ERR_WORKSPACE;
-  if (!all_aligned16(src_a, src_b, sink)) return LLMHIP_ERR_INVALID_ARG;
-  if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;
-  return from_hip(launch_stream_read(src_a, src_b, bytes_each, sink, variant, static_cast<hipStream_t>(stream)));
 }
 int llmhip_set_device(int device) {
   if (llmhip_device_count() < 1) return LLMHIP_ERR_NO_DEVICE;

@@ -25,7 +25,6 @@ SYMBOLS = {
     "llmhip_flash_attn": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_attn_gqa": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_attn_scratch_bytes": (_sz, [_i, _i, _i, _i, _i]),
-    "llmhip_flash_attn_gqa_clocked": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "llmhip_flash_attn_opt_prefill": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_gqa": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i64, _i, _i, _i, _i, _i, _vp]),
     "llmhip_flash_decode_gqa_static": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i64, _i, _i, _i, _i, _i, _vp]),
@@ -41,8 +40,6 @@ SYMBOLS = {
     "llmhip_add": (_i, [_vp, _vp, _vp, ctypes.c_longlong, _i, _vp]),
     "llmhip_device_count": (_i, []),
     "llmhip_device_props": (_i, [_i, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_sz)]),
-    "llmhip_probe_mfma_ceiling": (_i, [_i, ctypes.c_double, ctypes.POINTER(ctypes.c_double)]),
-    "llmhip_probe_stream_read": (_i, [_vp, _vp, _sz, _vp, _sz, _i, _vp]),
     "llmhip_set_device": (_i, [_i]),
     "llmhip_malloc": (_i, [ctypes.POINTER(_vp), _sz]),
     "llmhip_free": (_i, [_vp]),
@@ -114,16 +111,6 @@ def hip_flash_attn_gqa_layer(output_dev, q_dev, k_dev, v_dev, m, n, offset, grou
     _check(lib.llmhip_flash_attn_gqa(_ptr(output_dev), _ptr(q_dev), _ptr(k_dev), _ptr(v_dev), m,
                                      n, offset, group_size, kv_head_num, head_dim, dt, stream),
            "hip_flash_attn_gqa_layer")
-
-
-def hip_flash_attn_gqa_clocked_layer(output_dev, q_dev, k_dev, v_dev, m, n, offset, group_size,
-                                     kv_head_num, head_dim, dt, clock_probe_dev, stream=0):
-    """hip_flash_attn_gqa_layer on the prefill kernel, which also stores {shader-clock ticks,
-    100 MHz reference ticks} of its first workgroup at clock_probe_dev (two int64)."""
-    _check(lib.llmhip_flash_attn_gqa_clocked(_ptr(output_dev), _ptr(q_dev), _ptr(k_dev), _ptr(v_dev),
-                                             m, n, offset, group_size, kv_head_num, head_dim, dt,
-                                             _ptr(clock_probe_dev), stream),
-           "hip_flash_attn_gqa_clocked_layer")
 
 
 def hip_flash_attn_opt_prefill_layer(output_dev, q_dev, k_dev, v_dev, m, n, offset, head_num,
@@ -228,27 +215,6 @@ def device_props(device=0):
     _check(lib.llmhip_device_props(device, ctypes.byref(cus), ctypes.byref(khz), ctypes.byref(mem)),
            "device_props")
     return cus.value, khz.value / 1e3, mem.value
-
-
-def probe_mfma_ceiling(mix, target_ms=60.0):
-    """Sustained bf16 MFMA TFLOP/s on N(0,1) operands: mix 0 = MFMAs alone, mix 1 = with the LDS reads and
-    vector instructions of an attention inner loop beside them."""
-    t = ctypes.c_double(0.0)
-    _check(lib.llmhip_probe_mfma_ceiling(mix, float(target_ms), ctypes.byref(t)), "probe_mfma_ceiling")
-    return t.value
-
-
-STREAM_READ_SINK_BYTES = 65536
-
-
-def probe_stream_read(a, b, sink, variant, stream=None):
-    """Enqueues a plain streaming read of the two equally sized device tensors a and b (a measurement aid:
-    what a kernel that only reads gets from the memory system)."""
-    nbytes = a.numel() * a.element_size()
-    if b.numel() * b.element_size() != nbytes:
-        raise ValueError("probe_stream_read: a and b must have the same size")
-    _check(lib.llmhip_probe_stream_read(_ptr(a), _ptr(b), nbytes, _ptr(sink), sink.numel() * sink.element_size(),
-                                        variant, stream), "probe_stream_read")
 
 
 def _bf16_round_trip(x):

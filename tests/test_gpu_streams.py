@@ -88,35 +88,36 @@ def test_graph_capture_and_replay():
 
 
 def test_measurement_aids():
-    """The clocked prefill entry returns the same output as the plain one and plausible counters; the MFMA
+    """Measurement library (libllmhip_bench.so): the clocked prefill entry returns the same output as the plain one and plausible counters; the MFMA
     ceiling probe returns a rate between a tenth of the published peak and the peak."""
     import torch
+    import llm_simple_amd.bench_ops as bops
     import llm_simple_amd.ops as ops
     dt, S, H, Hkv = DT_BFLOAT16, 512, 8, 2
     q, k, v = (to_dev(normal_bits(s, (S, h, 128), dt)) for s, h in ((21, H), (22, Hkv), (23, Hkv)))
     o_a, o_b = dev_empty((S, H, 128)), dev_empty((S, H, 128))
     probe = torch.zeros(2, dtype=torch.int64, device="cuda")
     ops.hip_flash_attn_gqa_layer(o_a, q, k, v, S, S, 0, H // Hkv, Hkv, 128, dt)
-    ops.hip_flash_attn_gqa_clocked_layer(o_b, q, k, v, S, S, 0, H // Hkv, Hkv, 128, dt, probe)
+    bops.hip_flash_attn_gqa_clocked_layer(o_b, q, k, v, S, S, 0, H // Hkv, Hkv, 128, dt, probe)
     torch.cuda.synchronize()
     assert np.array_equal(to_host(o_a), to_host(o_b))
     ticks, ref = (int(x) for x in probe.cpu())
     assert ticks > 0 and ref > 0 and 300.0 < ticks / ref * 100.0 < 3000.0   # MHz
     # decode-sized shapes are refused by the clocked entry (it times the prefill kernel only)
-    assert ops.lib.llmhip_flash_attn_gqa_clocked(o_b.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), 1, S,
+    assert bops.lib.llmhip_bench_flash_attn_gqa_clocked(o_b.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), 1, S,
                                                  S - 1, H // Hkv, Hkv, 128, dt, probe.data_ptr(), None) == -2
-    alone, mix = ops.probe_mfma_ceiling(0, 5.0), ops.probe_mfma_ceiling(1, 5.0)
+    alone, mix = bops.probe_mfma_ceiling(0, 5.0), bops.probe_mfma_ceiling(1, 5.0)
     assert 250.0 < mix < alone < 2600.0, (alone, mix)
     cus, mhz, mem = ops.device_props(0)
     assert cus >= 64 and 1000.0 <= mhz <= 3000.0 and mem > (16 << 30)
 
 
 def test_plain_read_probe_reads_every_byte():
-    """llmhip_probe_stream_read XORs everything it reads into one word per wave: the XOR of those words must be
+    """llmhip_bench_stream_read XORs everything it reads into one word per wave: the XOR of those words must be
     the XOR of all 32-bit words of both arrays, for both launch shapes and a size that is not a multiple of the
     grid's stride."""
     import torch
-    import llm_simple_amd.ops as ops
+    import llm_simple_amd.bench_ops as bops
     rng = np.random.default_rng(5)
     for n_words in (4 * 1000, 4 * 262144 + 4 * 37):
         a = rng.integers(0, 2 ** 32, n_words, dtype=np.uint32)
@@ -124,8 +125,8 @@ def test_plain_read_probe_reads_every_byte():
         want = int(np.bitwise_xor.reduce(a) ^ np.bitwise_xor.reduce(b))
         d_a, d_b = to_dev(a.view(np.uint16)), to_dev(b.view(np.uint16))
         for variant in (0, 1):
-            sink = torch.zeros(ops.STREAM_READ_SINK_BYTES // 4, dtype=torch.int32, device="cuda")
-            ops.probe_stream_read(d_a, d_b, sink, variant)
+            sink = torch.zeros(bops.STREAM_READ_SINK_BYTES // 4, dtype=torch.int32, device="cuda")
+            bops.probe_stream_read(d_a, d_b, sink, variant)
             torch.cuda.synchronize()
             got = int(np.bitwise_xor.reduce(sink.cpu().numpy().view(np.uint32)))
             assert got == want, (n_words, variant, hex(got), hex(want))

@@ -10,8 +10,8 @@ import subprocess
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _header_symbols():
-    text = open(os.path.join(ROOT, "include", "llmhip.h")).read()
+def _header_symbols(header="llmhip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return set(re.findall(r"\b(llmhip_\w+)\s*\(", text))
 
@@ -23,6 +23,32 @@ def test_library_exports_every_declared_symbol():
     handle = ctypes.CDLL(ops.LIB_PATH)
     for name in declared:
         assert hasattr(handle, name), name
+
+
+def test_measurement_library_is_separate():
+    """The measurement aids live in libllmhip_bench.so / llmhip_bench.h: the product library exports none
+    of them, the measurement library exports exactly what its header declares, and validates arguments
+    before touching a device."""
+    import llm_simple_amd.bench_ops as bops
+    import llm_simple_amd.ops as ops
+    declared = _header_symbols("llmhip_bench.h")
+    assert declared == set(bops.SYMBOLS), declared ^ set(bops.SYMBOLS)
+    product = ctypes.CDLL(ops.LIB_PATH)
+    for name in declared:
+        assert hasattr(bops.lib, name), name
+        assert not hasattr(product, name), name
+    exported = subprocess.run(["nm", "-D", "--defined-only", ops.LIB_PATH], capture_output=True, text=True,
+                              check=True).stdout
+    assert "probe" not in exported and "clocked" not in exported and "ceiling" not in exported
+    buf = ctypes.create_string_buffer(96)
+    p = (ctypes.addressof(buf) + 15) & ~15
+    # the plain-read probe: size a multiple of 16, sink of the declared size, aligned pointers
+    assert bops.lib.llmhip_bench_stream_read(p, p, 24, p, bops.STREAM_READ_SINK_BYTES, 0, None) == -1
+    assert bops.lib.llmhip_bench_stream_read(p, p, 32, p, 1024, 0, None) == -3
+    assert bops.lib.llmhip_bench_stream_read(p, p + 4, 32, p, bops.STREAM_READ_SINK_BYTES, 0, None) == -1
+    assert bops.lib.llmhip_bench_stream_read(p, p, 32, p, bops.STREAM_READ_SINK_BYTES, 2, None) == -1
+    assert bops.lib.llmhip_bench_flash_attn_gqa_clocked(p, p, p, p, 1, 64, 63, 1, 1, 128, 5, p, None) == -2
+    assert bops.lib.llmhip_bench_mfma_ceiling(2, 1.0, None) == -1
 
 
 def test_cpp_overloads_cover_reference_operator_names():
@@ -51,11 +77,6 @@ def test_argument_validation_without_gpu():
     assert lib.llmhip_rope_single(p, p + 4, p, 0, 1, 2, 256, 0, 4, None) == -1
     assert lib.llmhip_rope_kv_append(p, p, p + 6, p, p, p, p, 0, 1, 1, 1, 128, 0, 4, None) == -1
     assert lib.llmhip_flash_decode_gqa_static(p, p, p + 2, p, 1, 16, 16, 5, 8, 128, 1, 5, None) == -1
-    # the plain-read probe: size a multiple of 16, sink of the declared size, aligned pointers
-    assert lib.llmhip_probe_stream_read(p, p, 24, p, ops.STREAM_READ_SINK_BYTES, 0, None) == -1
-    assert lib.llmhip_probe_stream_read(p, p, 32, p, 1024, 0, None) == -3
-    assert lib.llmhip_probe_stream_read(p, p + 4, 32, p, ops.STREAM_READ_SINK_BYTES, 0, None) == -1
-    assert lib.llmhip_probe_stream_read(p, p, 32, p, ops.STREAM_READ_SINK_BYTES, 2, None) == -1
     # the fused decode step: group size within the kernel's 16 columns, position not negative
     assert lib.llmhip_decode_step_gqa(p, p, p, p, p, p, p, 0, 17, 1, 128, 0, 5, None) == -2
     assert lib.llmhip_decode_step_gqa(p, p, p, p, p, p, p, -1, 5, 8, 128, 0, 5, None) == -1

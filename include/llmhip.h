@@ -33,6 +33,7 @@ extern "C" {
 #define LLMHIP_ERR_UNSUPPORTED (-2)   /* head_dim != 128, group too large for the kernel */
 #define LLMHIP_ERR_WORKSPACE (-3)     /* workspace missing or too small */
 #define LLMHIP_ERR_NO_DEVICE (-4)     /* no HIP device visible */
+#define LLMHIP_NOT_READY (-5)         /* llmhip_event_query: the event has not completed yet (no error) */
 
 /* Every device pointer handed to the operators below must be 16-byte aligned (anything the
  * runtime's allocator returns is; so is any row of a cache whose base is): the kernels move
@@ -70,9 +71,11 @@ int llmhip_flash_attn_opt_prefill(void *out, const void *q, const void *k, const
  * partials of the split-KV decode kernel (m * group_size <= 16) or of a key-range split of the
  * prefill kernel (a chunk of few rows over a cache at least 8 times longer); 0 for ordinary
  * prefill shapes.  The buffer is allocated on the first call that needs it on a stream (at least
- * 4 MiB), grows when a later call needs more, and is freed by llmhip_stream_destroy or
- * llmhip_release_internal_workspace: a caller that must not see an allocation later warms the
- * stream up with its largest shape. */
+ * 4 MiB) and replaced by a larger one when a later call needs more; a replaced buffer is kept, not
+ * freed, so launches already queued and HIP graphs captured earlier keep a valid pointer.  All of
+ * them go with llmhip_stream_destroy or llmhip_release_internal_workspace.  HIP graphs: a call made
+ * while its stream is capturing cannot allocate and is refused with LLMHIP_ERR_WORKSPACE when the
+ * buffer would have to grow -- warm the stream up with its largest shape before capturing. */
 size_t llmhip_flash_attn_scratch_bytes(int m, int n, int offset, int group_size, int kv_head_num);
 
 /* Batched split-KV decode over a contiguous per-sequence KV cache: one query
@@ -194,6 +197,10 @@ int llmhip_event_create(void **event);
 int llmhip_event_destroy(void *event);
 int llmhip_event_record(void *event, void *stream);
 int llmhip_event_sync(void *event);
+/* LLMHIP_OK once everything queued before the event's record has completed, LLMHIP_NOT_READY
+ * before that; never blocks (hipEventQuery).  The device layer's stream-ordered pool asks this
+ * before it hands a block freed on one stream to another. */
+int llmhip_event_query(void *event);
 int llmhip_event_elapsed_ms(float *ms, void *start, void *stop);
 const char *llmhip_error_string(int status);
 /* Frees the split-KV scratch the reference-signature attention entry points

@@ -7,6 +7,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <fstream>
+#include <tuple>
 #include <map>
 #include <memory>
 #include <string>
@@ -24,41 +25,90 @@ class CPUAllocator {
   static void Deallocate(void *ptr);
 };
 
-// Pooling device allocator with the contract of the reference's NPUAllocator
-// (src/device_npu.cpp:26-67): Allocate takes the smallest cached block that is
-// large enough, else asks the device and then, while more than dev_mem_max
-// bytes are owned, gives cached blocks back smallest first; Deallocate returns
-// a block to the cache.  Not thread safe, and -- as in the reference -- a
-// freed block can be handed out again at once, so the caller drains the stream
-// before temporaries go out of scope (src/llama2_layer_npu.cpp:605-608).
+// Pooling device allocator with the pooling contract of the reference's NPUAllocator
+// (src/device_npu.cpp:26-67): Allocate takes the smallest cached block that is large enough, else
+// asks the device and then, while more than dev_mem_max bytes are owned, gives cached blocks back
+// smallest first; Deallocate returns a block to the cache.
+//
+// Unlike the reference's pool this one is stream-ordered.  In the reference a freed block can be
+// handed out again at once, so every layer drains its stream before its temporaries go out of scope
+// (src/llama2_layer_npu.cpp:605-608, :990-993): one host round trip per layer per token.  Here a
+// block that is freed remembers the stream whose queued work may still touch it and a ticket of that
+// stream.  A request that names the same stream may take the block at once (its new use is queued
+// behind the old one); any other request -- another stream, or host code that names none -- gets it
+// only once an event recorded on that stream after the free has completed.  Such an event is recorded
+// when a request first needs it, not at every free, so a model that runs on one stream makes no event
+// call at all.  A block freed without a stream (never handed to a launch, or whose user drained the
+// stream itself) is free for everybody.  Not thread safe, like the reference's.
 class GPUAllocator {
  public:
   using RawAlloc = int (*)(void **, size_t);
   using RawFree = int (*)(void *);
+  // event backend: create / record on a stream / query (0 = complete, anything else = not yet) /
+  // wait / destroy; by default the llmhip_event_* calls of the C ABI
+  struct EventBackend {
+    int (*create)(void **event);
+    int (*record)(void *event, void *stream);
+    int (*query)(void *event);
+    int (*sync)(void *event);
+    int (*destroy)(void *event);
+    int (*device_sync)();
+  };
+  // Stream tags of a block: kNoStream = no queued work touches it; kAnyStream = some stream does but
+  // the caller did not say which (only a drained device makes it reusable).
+  static gpuStream_t NoStream() { return reinterpret_cast<gpuStream_t>(static_cast<uintptr_t>(1)); }
+  static gpuStream_t AnyStream() { return reinterpret_cast<gpuStream_t>(static_cast<uintptr_t>(2)); }
 
   static GPUAllocator &GetInstance();
-  static void *Allocate(size_t size);
-  static void Deallocate(void *ptr);
+  // stream: the stream the block will be used on (nullptr is the default stream, a stream like any
+  // other), or NoStream() for a request from host code that will touch the block with blocking calls.
+  static void *Allocate(size_t size, gpuStream_t stream = NoStream());
+  // stream: the stream whose queued work may still read or write the block, NoStream() if none can,
+  // AnyStream() if unknown.
+  static void Deallocate(void *ptr, gpuStream_t stream = NoStream());
 
-  // Test hooks: replace the device calls (default llmhip_malloc / llmhip_free)
-  // and the 8 GiB trim threshold; ReleaseAll frees every cached block.
+  // Test hooks: replace the device calls (default llmhip_malloc / llmhip_free, llmhip_event_*)
+  // and the 8 GiB trim threshold; ReleaseAll frees every cached block (after draining the device
+  // when any is still pending).
   void SetBackend(RawAlloc a, RawFree f);
+  void SetEventBackend(const EventBackend *b);
   void SetByteCap(size_t cap) { dev_mem_max_ = cap; }
   void ReleaseAll();
+  // Before a stream is destroyed: drain it, then tell the pool, which frees its blocks for everybody
+  // (a later stream may get the same handle).
+  void ForgetStream(gpuStream_t stream);
   size_t OwnedBytes() const { return owned_bytes_; }
   size_t CachedBlocks() const { return cache_.size(); }
+  size_t PendingBlocks() const;
+  size_t FenceEvents() const { return fence_events_; }  // events recorded so far (a single-stream model: 0)
 
  private:
+  struct Block {
+    void *ptr;
+    gpuStream_t stream;  // NoStream(): free for everybody
+    uint64_t ticket;     // position in that stream's sequence of frees
+  };
+  struct StreamState {
+    uint64_t next_ticket{1};   // ticket of the next free on this stream
+    uint64_t fenced{0};        // frees up to this ticket are covered by `event`
+    uint64_t completed{0};     // frees up to this ticket are known complete
+    void *event{nullptr};
+  };
   GPUAllocator();
-  void *AllocateImpl(size_t size);
-  void DeallocateImpl(void *ptr);
+  void *AllocateImpl(size_t size, gpuStream_t stream);
+  void DeallocateImpl(void *ptr, gpuStream_t stream);
+  bool Usable(const Block &b, gpuStream_t requester, bool may_wait);
+  void DrainAll();
 
-  std::multimap<size_t, void *> cache_;         // free blocks by size
+  std::multimap<size_t, Block> cache_;           // free and pending blocks by size
   std::unordered_map<void *, size_t> ptr_size_;  // every block this allocator owns
+  std::unordered_map<gpuStream_t, StreamState> streams_;
   size_t dev_mem_max_{8ULL << 30};
   size_t owned_bytes_{0};
+  size_t fence_events_{0};
   RawAlloc raw_alloc_;
   RawFree raw_free_;
+  EventBackend ev_;
 };
 
 // src/device.hpp:41-55.  data_size counts elements, bytes = SizeOfTensor().
@@ -67,7 +117,14 @@ class Tensor : public std::enable_shared_from_this<Tensor> {
   Tensor() = default;
   ~Tensor();
   static std::shared_ptr<Tensor> MakeCPUTensor(size_t size, DataType dtype);
-  static std::shared_ptr<Tensor> MakeGPUTensor(size_t size, DataType dtype);
+  // stream: the stream whose launches will use the tensor (the pool is stream-ordered, see
+  // GPUAllocator); without one the block comes from what no queued work can touch.
+  static std::shared_ptr<Tensor> MakeGPUTensor(size_t size, DataType dtype,
+                                               gpuStream_t stream = GPUAllocator::NoStream());
+  // Tells the tensor that work queued on `stream` reads or writes it, so that its block is not
+  // handed to anybody else before that work is done.  Layers call it on every tensor they pass
+  // to a launch; a tensor used on two different streams is kept until the device has drained.
+  void RecordStream(gpuStream_t stream);
 
   // Same device: this tensor; other device: a new tensor filled by a blocking
   // copy (src/device.cpp:22-52).
@@ -78,6 +135,7 @@ class Tensor : public std::enable_shared_from_this<Tensor> {
   size_t data_size{0};
   DataType data_type{DT_FLOAT16};
   DeviceType dev_type{DEV_CPU};
+  gpuStream_t stream_tag{GPUAllocator::NoStream()};  // see RecordStream
 };
 
 // Chrome-trace ("chrome://tracing", Perfetto) writer of the reference's profiler
@@ -128,11 +186,16 @@ class AppProfileGuard {
   ::llm_simple_amd::AppProfileGuard LLM_AMD_CONCAT(temp_perf_obj_, __LINE__)(                    \
       name, info, stream, profiler, __FILE__, __LINE__, isprofiling)
 
+class ModelBase;
+
 // Positions of one step (src/model_base.hpp:40-48): cur_size = cur_pos - prev_pos
 // query tokens, keys [0, cur_pos) valid after the append.
 struct InferenceCtx {
   InferenceCtx(size_t cur_pos_, size_t prev_pos_, gpuStream_t stream = nullptr)
       : cur_pos(cur_pos_), prev_pos(prev_pos_), cur_size(cur_pos_ - prev_pos_), gpu_stream(stream) {}
+  // the reference's constructor (src/model_base.hpp:42); stream, profiler and profiling flag come from the model
+  InferenceCtx(ModelBase *model, size_t cur_pos_, size_t prev_pos_);
+  ModelBase *model{nullptr};
   size_t cur_pos;
   size_t prev_pos;
   size_t cur_size;
@@ -158,6 +221,9 @@ class AttentionGPUImpl {
  public:
   bool Init(int n_heads, int n_kv_heads, int head_dim, int max_seq_len, DataType dtype,
             bool rope_is_neox_style, std::shared_ptr<Tensor> freq_cis_gpu);
+  // the same with the rotary table as a bare device pointer that somebody else owns (ModelBase::freq_cis)
+  bool Init(int n_heads, int n_kv_heads, int head_dim, int max_seq_len, DataType dtype,
+            bool rope_is_neox_style, float *freq_cis_dev);
   // q: [cur_size][n_heads*head_dim], k, v: [cur_size][n_kv_heads*head_dim], on the GPU.
   // Returns [cur_size][n_heads*head_dim].  Asynchronous on ctx.gpu_stream.
   std::shared_ptr<Tensor> Forward(std::shared_ptr<Tensor> q, std::shared_ptr<Tensor> k,
@@ -168,7 +234,8 @@ class AttentionGPUImpl {
   int n_heads_{0}, n_kv_heads_{0}, head_dim_{0}, max_seq_len_{0};
   DataType dtype_{DT_FLOAT16};
   bool neox_{false};
-  std::shared_ptr<Tensor> freq_cis_;
+  float *freqs_cis_{nullptr};
+  std::shared_ptr<Tensor> freq_cis_owner_;
 };
 
 // Dense projection y = x W^T (+ bias) on the GPU: MatmulLayerNPUImpl without quantisation
@@ -209,6 +276,153 @@ class AttentionBlockGPUImpl {
  private:
   int hidden_dim_{0};
   DataType dtype_{DT_FLOAT16};
+};
+
+// ---------------------------------------------------------------------------
+// Device dispatch: the layer facades of the reference (src/model_base.hpp, src/model_base.cpp)
+// for the layers on this path, with the DEV_GPU arm that the reference leaves out.
+// ---------------------------------------------------------------------------
+
+// What these layers read of the reference's ModelConfig (src/model_base.hpp:18-36) ...
+class ModelConfig {
+ public:
+  DeviceType device_type{DEV_GPU};
+  DataType data_type{DT_FLOAT16};
+  int max_seq_len{2048};
+  bool rope_is_neox_style{false};
+  bool debug_print{false};
+};
+
+// ... and of ModelBase (src/model_base.hpp:324-354): dimensions, the model's one stream, the
+// rotary table and the profiler.
+class ModelBase {
+ public:
+  virtual ~ModelBase() = default;
+  // src/model_base.cpp:27-83 with the device arm for DEV_GPU: the table is built on the host and,
+  // for DEV_GPU, copied to the device once; freq_cis then is a device pointer.
+  bool InitFreqCIS(const float theta = 10000.0f, const DataType dt = DT_FLOAT32);
+
+  ModelConfig config;
+  int hidden_dim{0};
+  int head_dim{0};
+  int n_heads{0};
+  int n_kv_heads{0};
+  gpuStream_t model_stream{nullptr};
+  float *freq_cis{nullptr};
+  bool is_profiling{false};
+  AppProfiler profiler;
+
+ private:
+  std::shared_ptr<Tensor> freq_cis_holder_;
+};
+
+// src/model_base.hpp:106-133.
+class RoPELayerImpl {
+ public:
+  virtual ~RoPELayerImpl();
+  virtual std::tuple<std::shared_ptr<Tensor>, std::shared_ptr<Tensor>> Forward(std::shared_ptr<Tensor> input_q,
+                                                                              std::shared_ptr<Tensor> input_k,
+                                                                              InferenceCtx &ctx) = 0;
+  virtual bool Init(ModelBase *model, const std::string &weight_path);
+  virtual void UnInit();
+
+  size_t hidden_dim{0};
+  size_t n_heads{0};
+  size_t head_dim{0};
+  size_t rope_dim{0};
+  size_t weight_size{0};
+  bool rope_is_neox_style{false};
+  DataType dtype{DT_FLOAT16};
+  float *freqs_cis{nullptr};
+};
+
+// The GPU sibling of RoPELayerNPUImpl (src/llama2_layer_npu.cpp:183-222): q and k of the same head
+// count rotated by one hip_rope_layer call, outputs from the pool.
+class RoPELayerGPUImpl : public RoPELayerImpl {
+ public:
+  ~RoPELayerGPUImpl() override;
+  std::tuple<std::shared_ptr<Tensor>, std::shared_ptr<Tensor>> Forward(std::shared_ptr<Tensor> input_q,
+                                                                      std::shared_ptr<Tensor> input_k,
+                                                                      InferenceCtx &ctx) override;
+  bool Init(ModelBase *model, const std::string &weight_path) override;
+};
+
+class RoPELayer {
+ public:
+  ~RoPELayer();
+  std::tuple<std::shared_ptr<Tensor>, std::shared_ptr<Tensor>> Forward(std::shared_ptr<Tensor> input_q,
+                                                                      std::shared_ptr<Tensor> input_k,
+                                                                      InferenceCtx &ctx);
+  // src/model_base.cpp:620-635: picks the implementation by model->config.device_type.
+  bool Init(ModelBase *model, const std::string &weight_path);
+  void UnInit();
+  RoPELayerImpl *impl{nullptr};
+};
+
+// The attention part of a transformer layer -- between the q/k/v projections and o_proj -- behind
+// the same kind of facade as the reference's Llamma2TransformerLayer / Qwen2TransformerLayer
+// (src/model_base.hpp; the rest of those layers, norms and FFN, is outside this path).
+class AttentionLayerImpl {
+ public:
+  virtual ~AttentionLayerImpl();
+  // q [cur_size][n_heads*head_dim], k, v [cur_size][n_kv_heads*head_dim] on the device, unrotated;
+  // returns [cur_size][n_heads*head_dim].
+  virtual std::shared_ptr<Tensor> Forward(std::shared_ptr<Tensor> q, std::shared_ptr<Tensor> k,
+                                          std::shared_ptr<Tensor> v, InferenceCtx &ctx) = 0;
+  virtual bool Init(ModelBase *model, int layer_no);
+  virtual void UnInit();
+
+  size_t hidden_dim{0};
+  size_t head_dim{0};
+  size_t n_heads{0};
+  size_t n_kv_heads{0};
+  size_t max_seq_len{0};
+  DataType dtype{DT_FLOAT16};
+  std::shared_ptr<Tensor> k_cache, v_cache;
+};
+
+// Llama-2 on the GPU, call for call what Llamma2TransformerLayerNPUImpl::Forward does
+// (src/llama2_layer_npu.cpp:284, :325-339, :370-374): rope_emb.Forward, two device-to-device copies
+// into the caches, hip_flash_attn_opt_prefill_layer.  n_kv_heads == n_heads.
+class Llama2AttentionGPUImpl : public AttentionLayerImpl {
+ public:
+  std::shared_ptr<Tensor> Forward(std::shared_ptr<Tensor> q, std::shared_ptr<Tensor> k, std::shared_ptr<Tensor> v,
+                                  InferenceCtx &ctx) override;
+  bool Init(ModelBase *model, int layer_no) override;
+  RoPELayer rope_emb;
+};
+
+// Qwen2 on the GPU (src/llama2_layer_npu.cpp:790-869): the fused operators of AttentionGPUImpl.
+class Qwen2AttentionGPUImpl : public AttentionLayerImpl {
+ public:
+  std::shared_ptr<Tensor> Forward(std::shared_ptr<Tensor> q, std::shared_ptr<Tensor> k, std::shared_ptr<Tensor> v,
+                                  InferenceCtx &ctx) override;
+  bool Init(ModelBase *model, int layer_no) override;
+
+ private:
+  AttentionGPUImpl impl_;
+};
+
+// src/model_base.cpp:248-264.
+class Llama2AttentionLayer {
+ public:
+  ~Llama2AttentionLayer();
+  std::shared_ptr<Tensor> Forward(std::shared_ptr<Tensor> q, std::shared_ptr<Tensor> k, std::shared_ptr<Tensor> v,
+                                  InferenceCtx &ctx);
+  bool Init(ModelBase *model, int layer_no);
+  void UnInit();
+  AttentionLayerImpl *impl{nullptr};
+};
+
+// src/model_base.cpp:294-306.
+class Qwen2AttentionLayer {
+ public:
+  ~Qwen2AttentionLayer();
+  std::shared_ptr<Tensor> Forward(std::shared_ptr<Tensor> q, std::shared_ptr<Tensor> k, std::shared_ptr<Tensor> v,
+                                  InferenceCtx &ctx);
+  bool Init(ModelBase *model, int layer_no);
+  void UnInit();
+  AttentionLayerImpl *impl{nullptr};
 };
 
 }  // namespace llm_simple_amd

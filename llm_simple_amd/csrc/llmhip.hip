@@ -7,6 +7,7 @@
 
 #include <map>
 #include <mutex>
+#include <vector>
 
 #include "kernels.hpp"
 
@@ -25,30 +26,32 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 template <typename... P> inline bool all_aligned16(P... ptrs) { return (aligned16(ptrs) && ...); }
 
 // Split-KV scratch for the entry points that mirror the reference signatures
-// and therefore have no workspace argument: one grow-only buffer per stream.
+// and therefore have no workspace argument: one buffer per stream that only grows.
+// A buffer that has become too small is not freed when a larger one replaces it: launches already
+// queued, and HIP graphs captured earlier, keep their pointer valid.  Retired buffers go with
+// llmhip_stream_destroy / llmhip_release_internal_workspace.
 struct StreamScratch {
   void *ptr = nullptr;
   size_t bytes = 0;
+  std::vector<void *> retired;
 };
 std::mutex g_scratch_mu;
 std::map<void *, StreamScratch> g_scratch;
 
-// Caller holds g_scratch_mu, and keeps holding it until the launch that uses the buffer is enqueued:
-// a second thread growing the same stream's buffer then cannot free it in between.
+// Caller holds g_scratch_mu.  Growing allocates, which a stream under capture must not do: such a
+// call is refused with LLMHIP_ERR_WORKSPACE (warm the stream up with its largest shape first).
 int scratch_for_locked(void *stream, size_t need, void **out) {
   StreamScratch &s = g_scratch[stream];
   if (s.bytes < need) {
-    if (s.ptr) {
-      // the old buffer may still be read by work queued on this stream
-      hipError_t e = hipStreamSynchronize(as_stream(stream));
-      if (e != hipSuccess) return (int)e;
-      (void)hipFree(s.ptr);
-      s.ptr = nullptr;
-      s.bytes = 0;
-    }
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(as_stream(stream), &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone) return LLMHIP_ERR_WORKSPACE;
     size_t want = need < (size_t)(4u << 20) ? (size_t)(4u << 20) : need;
-    hipError_t e = hipMalloc(&s.ptr, want);
+    void *fresh = nullptr;
+    hipError_t e = hipMalloc(&fresh, want);
     if (e != hipSuccess) return (int)e;
+    if (s.ptr) s.retired.push_back(s.ptr);
+    s.ptr = fresh;
     s.bytes = want;
   }
   *out = s.ptr;
@@ -316,6 +319,7 @@ int llmhip_stream_destroy(void *stream) {
         (void)hipStreamSynchronize(as_stream(stream));
         (void)hipFree(it->second.ptr);
       }
+      for (void *old : it->second.retired) (void)hipFree(old);
       g_scratch.erase(it);
     }
   }
@@ -341,6 +345,14 @@ int llmhip_event_record(void *event, void *stream) {
 int llmhip_event_sync(void *event) {
   return from_hip(hipEventSynchronize(static_cast<hipEvent_t>(event)));
 }
+int llmhip_event_query(void *event) {
+  const hipError_t e = hipEventQuery(static_cast<hipEvent_t>(event));
+  if (e == hipErrorNotReady) {
+    (void)hipGetLastError();  // not an error: leave nothing behind for the next call to report
+    return LLMHIP_NOT_READY;
+  }
+  return from_hip(e);
+}
 int llmhip_event_elapsed_ms(float *ms, void *start, void *stop) {
   if (!ms) return LLMHIP_ERR_INVALID_ARG;
   return from_hip(
@@ -355,6 +367,7 @@ const char *llmhip_error_string(int status) {
       return "workspace missing or too small (or batch * kv heads * splits beyond the fixed scratch of the "
              "allocation-free decode)";
     case LLMHIP_ERR_NO_DEVICE: return "no HIP device";
+    case LLMHIP_NOT_READY: return "event not complete yet";
     default: break;
   }
   if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -373,6 +386,7 @@ int llmhip_release_internal_workspace(void) {
       hipError_t e = hipFree(kv.second.ptr);
       if (e != hipSuccess) rc = (int)e;
     }
+    for (void *old : kv.second.retired) (void)hipFree(old);
   }
   g_scratch.clear();
   release_matmul_resources();

@@ -55,6 +55,7 @@ SYMBOLS = {
     "llmhip_event_destroy": (_i, [_vp]),
     "llmhip_event_record": (_i, [_vp, _vp]),
     "llmhip_event_sync": (_i, [_vp]),
+    "llmhip_event_query": (_i, [_vp]),
     "llmhip_event_elapsed_ms": (_i, [ctypes.POINTER(ctypes.c_float), _vp, _vp]),
     "llmhip_error_string": (ctypes.c_char_p, [_i]),
     "llmhip_release_internal_workspace": (_i, []),

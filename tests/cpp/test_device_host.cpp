@@ -87,6 +87,203 @@ static void test_allocator_pool() {
   a.SetByteCap(8ULL << 30);
 }
 
+// A fake event backend: an event completes when the test says so.  Records what the pool asked for.
+struct FakeEvent {
+  void *stream = nullptr;
+  bool recorded = false, complete = false;
+};
+static int g_ev_created = 0, g_ev_destroyed = 0, g_ev_records = 0, g_ev_syncs = 0, g_dev_syncs = 0;
+static std::vector<FakeEvent *> g_events;
+static int fake_create(void **e) {
+  auto *ev = new FakeEvent();
+  g_events.push_back(ev);
+  *e = ev;
+  ++g_ev_created;
+  return 0;
+}
+static int fake_record(void *e, void *stream) {
+  auto *ev = static_cast<FakeEvent *>(e);
+  ev->stream = stream;
+  ev->recorded = true;
+  ev->complete = false;
+  ++g_ev_records;
+  return 0;
+}
+static int fake_query(void *e) { return static_cast<FakeEvent *>(e)->complete ? 0 : LLMHIP_NOT_READY; }
+static int fake_sync(void *e) {
+  static_cast<FakeEvent *>(e)->complete = true;  // waiting makes it complete
+  ++g_ev_syncs;
+  return 0;
+}
+static int fake_destroy(void *e) {
+  delete static_cast<FakeEvent *>(e);
+  ++g_ev_destroyed;
+  return 0;
+}
+static int fake_device_sync() {
+  ++g_dev_syncs;
+  return 0;
+}
+
+// The pool is stream-ordered: a block freed under work queued on one stream goes back to that
+// stream at once, and to anybody else only after an event of that stream has completed.
+static void test_allocator_stream_order() {
+  GPUAllocator &a = GPUAllocator::GetInstance();
+  const GPUAllocator::EventBackend fake = {fake_create, fake_record, fake_query, fake_sync, fake_destroy,
+                                           fake_device_sync};
+  a.SetBackend(host_alloc, host_free);
+  a.SetEventBackend(&fake);
+  a.SetByteCap(1 << 20);
+  g_allocs = g_frees = 0;
+  int sa = 0, sb = 0;  // two stream handles
+  gpuStream_t A = &sa, B = &sb;
+
+  // same stream: immediate reuse, no event at all
+  void *p = GPUAllocator::Allocate(4096, A);
+  GPUAllocator::Deallocate(p, A);
+  EXPECT(a.PendingBlocks() == 1);
+  void *p_again = GPUAllocator::Allocate(4096, A);
+  EXPECT(p_again == p && g_allocs == 1 && a.FenceEvents() == 0 && g_ev_records == 0);
+
+  // another stream while the first one's work is pending: the block is NOT reused, a fresh one is
+  // allocated, and an event now guards the pending block
+  GPUAllocator::Deallocate(p, A);
+  void *q = GPUAllocator::Allocate(4096, B);
+  EXPECT(q != p && g_allocs == 2 && a.FenceEvents() == 1 && g_ev_records == 1 && g_ev_syncs == 0);
+  EXPECT(!g_events.empty() && g_events.back()->stream == A);
+  // host code (no stream) is treated like another stream
+  void *h = GPUAllocator::Allocate(4096);
+  EXPECT(h != p && h != q && g_allocs == 3 && g_ev_records == 1);  // the event in flight already covers p
+  // once the event has completed the block is anybody's
+  g_events.back()->complete = true;
+  void *r = GPUAllocator::Allocate(4096, B);
+  EXPECT(r == p && g_allocs == 3);
+
+  // a block freed after the event was recorded is not covered by it
+  GPUAllocator::Deallocate(r, B);   // pending on B, ticket 1
+  GPUAllocator::Deallocate(q, B);   // pending on B, ticket 2
+  void *x = GPUAllocator::Allocate(4096, A);  // asks for B's blocks: records a fence on B (covers both)
+  EXPECT(x != r && x != q && g_allocs == 4 && g_ev_records == 2);
+  FakeEvent *fence_b = g_events.back();
+  EXPECT(fence_b->stream == B);
+  GPUAllocator::Deallocate(h, B);   // ticket 3: freed after the fence
+  fence_b->complete = true;
+  void *y1 = GPUAllocator::Allocate(4096, A), *y2 = GPUAllocator::Allocate(4096, A);
+  EXPECT((y1 == r || y1 == q) && (y2 == r || y2 == q) && y1 != y2 && g_allocs == 4);
+  void *y3 = GPUAllocator::Allocate(4096, A);  // only h is cached, and the completed fence does not cover it
+  EXPECT(y3 != h && g_allocs == 5 && g_ev_records == 3);
+
+  // at the byte cap the pool waits for a pending block instead of allocating
+  a.SetByteCap(a.OwnedBytes());
+  const int syncs_before = g_ev_syncs;
+  void *w = GPUAllocator::Allocate(4096);
+  EXPECT(w == h && g_allocs == 5 && g_ev_syncs == syncs_before + 1);
+  a.SetByteCap(1 << 20);
+
+  // a block whose user did not name its stream comes back only after the device has drained
+  GPUAllocator::Deallocate(w, GPUAllocator::AnyStream());
+  void *z = GPUAllocator::Allocate(4096, A);
+  EXPECT(z != w && g_dev_syncs == 0);
+  a.SetByteCap(a.OwnedBytes());
+  void *z2 = GPUAllocator::Allocate(4096, A);
+  EXPECT(z2 == w && g_dev_syncs == 1);
+  a.SetByteCap(1 << 20);
+
+  // ForgetStream: a drained stream's blocks are free for everybody
+  GPUAllocator::Deallocate(z2, A);
+  a.ForgetStream(A);
+  EXPECT(a.PendingBlocks() == 0);
+  EXPECT(GPUAllocator::Allocate(4096, B) == z2);
+
+  // Tensor tags: born with the stream it was allocated for, one stream stays, two become "any"
+  {
+    auto t = Tensor::MakeGPUTensor(16, DT_FLOAT16);
+    EXPECT(t->stream_tag == GPUAllocator::NoStream());
+    t->RecordStream(A);
+    EXPECT(t->stream_tag == A);
+    t->RecordStream(A);
+    EXPECT(t->stream_tag == A);
+    t->RecordStream(B);
+    EXPECT(t->stream_tag == GPUAllocator::AnyStream());
+    auto u = Tensor::MakeGPUTensor(16, DT_FLOAT16, B);
+    EXPECT(u->stream_tag == B);
+  }
+  EXPECT(a.PendingBlocks() == 2);
+  for (void *blk : {z2, z, y1, y2, y3, x}) GPUAllocator::Deallocate(blk);
+  a.ReleaseAll();
+  EXPECT(a.OwnedBytes() == 0 && g_ev_created == g_ev_destroyed);
+  a.SetEventBackend(nullptr);
+  a.SetBackend(nullptr, nullptr);
+  a.SetByteCap(8ULL << 30);
+}
+
+// The layer facades pick their implementation by model->config.device_type
+// (src/model_base.cpp:248-264, :294-306, :620-635): the GPU arm exists, everything else is refused.
+namespace {
+struct TestModel : ModelBase {};
+}  // namespace
+static void test_device_dispatch() {
+  GPUAllocator &a = GPUAllocator::GetInstance();
+  a.SetBackend(host_alloc, host_free);  // cache tensors come from the host in this test
+  TestModel model;
+  model.hidden_dim = 4 * 128;
+  model.n_heads = 4;
+  model.n_kv_heads = 4;
+  model.head_dim = 128;
+  model.config.max_seq_len = 32;
+  model.config.data_type = DT_FLOAT16;
+  model.config.rope_is_neox_style = false;
+  float dummy_table[4] = {1, 0, 1, 0};
+  model.freq_cis = dummy_table;  // never dereferenced on the host
+  for (DeviceType dev : {DEV_CPU, DEV_NPU}) {
+    model.config.device_type = dev;
+    RoPELayer rope;
+    Llama2AttentionLayer llama;
+    Qwen2AttentionLayer qwen;
+    EXPECT(!rope.Init(&model, "") && rope.impl == nullptr);
+    EXPECT(!llama.Init(&model, 0) && llama.impl == nullptr);
+    EXPECT(!qwen.Init(&model, 0) && qwen.impl == nullptr);
+  }
+  model.config.device_type = DEV_GPU;
+  {
+    RoPELayer rope;
+    EXPECT(rope.Init(&model, "") && dynamic_cast<RoPELayerGPUImpl *>(rope.impl) != nullptr);
+    EXPECT(rope.impl->hidden_dim == 512 && rope.impl->n_heads == 4 && rope.impl->head_dim == 128 &&
+           rope.impl->freqs_cis == dummy_table && !rope.impl->rope_is_neox_style);
+    Llama2AttentionLayer llama;
+    EXPECT(llama.Init(&model, 0) && dynamic_cast<Llama2AttentionGPUImpl *>(llama.impl) != nullptr);
+    EXPECT(llama.impl->k_cache && llama.impl->k_cache->data_size == (size_t)32 * 512);
+    model.n_kv_heads = 2;
+    model.config.data_type = DT_BFLOAT16;
+    model.config.rope_is_neox_style = true;
+    Qwen2AttentionLayer qwen;
+    EXPECT(qwen.Init(&model, 0) && dynamic_cast<Qwen2AttentionGPUImpl *>(qwen.impl) != nullptr);
+    EXPECT(qwen.impl->n_kv_heads == 2 && qwen.impl->k_cache->data_size == (size_t)32 * 256);
+    // Llama-2 has as many kv heads as heads: the Llama sequence refuses a GQA model
+    Llama2AttentionLayer bad;
+    EXPECT(!bad.Init(&model, 0));
+    // positions that do not fit the cache are refused before anything is queued
+    auto t = Tensor::MakeGPUTensor(512, DT_BFLOAT16);
+    InferenceCtx past_end(33, 32, nullptr), inconsistent(8, 2, nullptr);
+    inconsistent.cur_size = 3;
+    EXPECT(qwen.Forward(t, t, t, past_end) == nullptr);
+    EXPECT(qwen.Forward(t, t, t, inconsistent) == nullptr);
+    // a head size the kernels do not take
+    model.hidden_dim = 4 * 64;
+    RoPELayer small;
+    EXPECT(!small.Init(&model, ""));
+  }
+  // the reference's context constructor takes stream and profiler from the model
+  int s = 0;
+  model.model_stream = &s;
+  model.is_profiling = true;
+  InferenceCtx ctx(&model, 10, 7);
+  EXPECT(ctx.model == &model && ctx.gpu_stream == &s && ctx.cur_size == 3 && ctx.profiler == &model.profiler &&
+         ctx.is_profiling);
+  a.ReleaseAll();
+  a.SetBackend(nullptr, nullptr);
+}
+
 static void test_tensor_cpu() {
   auto t = Tensor::MakeCPUTensor(16, DT_FLOAT32);
   EXPECT(t->dev_type == DEV_CPU && t->data_size == 16 && t->data_ptr != nullptr);
@@ -199,6 +396,8 @@ int main() {
   test_profiler_file();
   test_sizes();
   test_allocator_pool();
+  test_allocator_stream_order();
+  test_device_dispatch();
   test_tensor_cpu();
   test_freq_cis();
   test_abi_validation();

@@ -52,6 +52,37 @@ def test_attention_layer_prefill_then_decode(flags):
 
 
 @pytest.mark.parametrize("flags", [
+    # Llama2-7B, benchmark configurations 1 and 2 in one run: prefill 256, decode up to row 511
+    ("--model", "llama2", "--head_num", 32, "--kv_head_num", 32, "--prompt", 256, "--steps", 12, "--dtype", "fp16",
+     "--is_neox", 0, "--theta", 10000, "--max_seq_len", 512),
+    ("--model", "llama2", "--head_num", 8, "--kv_head_num", 8, "--prompt", 100, "--steps", 4, "--chunk", 40,
+     "--dtype", "bf16", "--is_neox", 1, "--max_seq_len", 256),
+])
+def test_llama_sequence_through_the_device_switch(flags):
+    """Llama2AttentionLayer (DEV_GPU arm of the layer switch): RoPELayer::Forward -> two device-to-device copies
+    -> hip_flash_attn_opt_prefill_layer, as src/llama2_layer_npu.cpp:284, :325-339, :370-374 issues them;
+    outputs and caches bit-identical to the fused path, and within tolerance of the oracle."""
+    out = _run("op_test_attention_layer", *flags)
+    assert "vs fused path: outputs bit-identical" in out and "caches bit-identical" in out, out
+
+
+def test_qwen_layer_through_the_device_switch_and_decode_loop_timing():
+    """Qwen2AttentionLayer behind the facade, checked; then the decode loop of benchmark configuration 3
+    (256 prompt tokens, 256 generated) timed through the layer: no host wait per step, no event of the pool."""
+    import json
+    _run("op_test_attention_layer", "--model", "qwen2", "--head_num", 12, "--kv_head_num", 2, "--prompt", 256,
+         "--steps", 16, "--dtype", "bf16", "--is_neox", 1)
+    exe = os.path.join(BIN, "op_test_attention_layer")
+    r = subprocess.run([exe, "--head_num", "12", "--kv_head_num", "2", "--prompt", "256", "--steps", "256",
+                        "--time", "3", "--dtype", "bf16"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    t = json.loads(r.stdout.strip().splitlines()[-1])
+    print(t, flush=True)
+    assert t["status"] == 0 and t["pool_fence_events"] == 0
+    assert 0 < t["layer_decode_us_per_step"] < 200 and 0 < t["abi_decode_us_per_step"] < 200
+
+
+@pytest.mark.parametrize("flags", [
     ("--m", 2048, "--n", 2048, "--k", 2048, "--dtype", "fp16"),                       # the reference CLI's defaults
     ("--m", 256, "--n", 3584, "--k", 3584, "--bias", 1, "--dtype", "bf16"),           # Qwen2.5-7B q_proj
     ("--m", 1, "--n", 512, "--k", 3584, "--bias", 1, "--dtype", "bf16"),              # k_proj, decode

@@ -367,7 +367,6 @@ __global__ __launch_bounds__(kDecThreads) void flash_decode_kernel(DecodeParams 
 // dims per thread, all of a thread's loads issued before any is used), then the 8 groups are merged
 // through LDS.  With few splits the surplus groups have nothing to load.
 constexpr int kMaxSplits = 256;
-constexpr int kDecTargetWgs = 256;  // workgroups of one round: the CUs of the part this is tuned on
 
 template <typename T>
 __global__ __launch_bounds__(256) void flash_decode_combine_kernel(DecodeParams p) {
@@ -440,38 +439,42 @@ __global__ __launch_bounds__(256) void flash_decode_combine_kernel(DecodeParams 
   *reinterpret_cast<u32x2_t *>(p.out + (((size_t)b * p.m + r) * p.H + kvh * p.g + hq) * kRowBytes + d4 * 8) = w;
 }
 
-// Largest split count the default rule considers for batch * kv heads = pairs (any KV length).
+// Largest split count the default rule considers for batch * kv heads = pairs (any KV length): one
+// round of workgroups, one workgroup per CU of the current device.
 int flash_decode_max_default_splits(long long pairs) {
-  long long base = (kDecTargetWgs + pairs - 1) / pairs;  // one round of workgroups
+  const long long cus = device_compute_units();
+  long long base = (cus + pairs - 1) / pairs;
   if (base < 8) base = 8;
   if (base > kMaxSplits) base = kMaxSplits;
   return (int)base;
 }
 
 // Split count that a simple model of the launch makes fastest.  Workgroups run one per CU in rounds
-// of kDecTargetWgs; a CU of a full round streams 25 GB/s (all of them together what the memory system
-// gives a reader, 6.4 TB/s), a CU of a thin round at most 31 GB/s; a workgroup costs 3 us beyond its
-// bytes, the combine launch 5 us.  Among the counts within 3 % of the best, one that fills its rounds
-// exactly is preferred, else the smallest.  For the common shapes this is about one workgroup per CU
-// (batch 16 x 8 kv heads -> 2 splits, batch 1 -> 32); for pair counts that do not divide a round it
-// finds the count that fills the rounds (model / measured us, n = 8192: batch 12, 1/2/3/5/8 splits ->
-// 138/76/115/75/77 against 133/80/106/76/76; batch 24, 1/2/4 -> 138/163/140 against 150/158/145;
-// batch 40, 1/2/3/4 -> measured 294/242/231/233).
-int flash_decode_default_splits(int batch, int n, int kv_head_num) {
-  const long long pairs = (long long)batch * kv_head_num;
-  const int nblocks = (n + kDecStepKeys - 1) / kDecStepKeys;
+// of as many workgroups as the device has CUs; a CU of a full round streams 27.7 GB/s (all 256 of an
+// MI355X together 7.1 TB/s, what its memory system gives a kernel that only reads), a CU of a thin
+// round at most 32 GB/s (one workgroup keeps 32 KiB of loads in flight); a workgroup costs 3 us beyond
+// its bytes, the combine launch 5 us.  Among the counts within 3 % of the best, one that fills its
+// rounds exactly is preferred, else the smallest.  For the common shapes this is about one workgroup
+// per CU (batch 16 x 8 kv heads -> 2 splits, batch 1 -> 32); for pair counts that do not divide a round
+// it finds the count that fills the rounds.  Model / measured us on 256 CUs, bf16, cold: batch 1,
+// n = 32768, 32 splits 26.9 / 26.2; batch 16, n = 4096, 2 splits 45.9 / 44.6; n = 8192: batch 12,
+// 5 splits 68.6 / 68.6, batch 20, 3 splits 108.5 / 107.6, batch 40, 4 splits 209.3 / 206.8, batch 48,
+// 2 splits 241.1 / 234.4 -- in a sweep of 38 shapes the count chosen is the fastest measured one or
+// within 1.6 % of it.
+static int default_splits_model(long long pairs, int nblocks, int cus) {
   int smax = flash_decode_max_default_splits(pairs);
   if (smax > nblocks) smax = nblocks;
   if (smax < 1) smax = 1;
   const double key_bytes = 2.0 * kRowBytes;  // K and V row of one kv head
+  const double all_cus = 27.7e9 * cus;       // what the memory system gives all CUs together
   auto model = [&](int s) {
     const long long wgs = pairs * s;
-    const long long full = wgs / kDecTargetWgs, rest = wgs % kDecTargetWgs;
+    const long long full = wgs / cus, rest = wgs % cus;
     const double wg_bytes = key_bytes * kDecStepKeys * ((nblocks + s - 1) / s);
-    double t = full * (wg_bytes / 25e9 + 3e-6);
+    double t = full * (wg_bytes / 27.7e9 + 3e-6);
     if (rest > 0) {
-      double rate = 6.4e12 / (double)rest;
-      if (rate > 31e9) rate = 31e9;
+      double rate = all_cus / (double)rest;
+      if (rate > 32e9) rate = 32e9;
       t += wg_bytes / rate + 3e-6;
     }
     return s > 1 ? t + 5e-6 : t;
@@ -485,9 +488,36 @@ int flash_decode_default_splits(int batch, int n, int kv_head_num) {
   for (int s = 1; s <= smax; ++s) {
     if (model(s) > t_min * 1.03) continue;
     if (first == 0) first = s;
-    if ((pairs * s) % kDecTargetWgs == 0) return s;
+    if ((pairs * s) % cus == 0) return s;
   }
   return first;
+}
+
+// The model is evaluated a few hundred times per call; a decode loop asks for the same (pairs, key
+// blocks) at every layer and for the next block count only every 128 tokens, so the last answers are
+// kept per thread.
+int flash_decode_default_splits(int batch, int n, int kv_head_num) {
+  const long long pairs = (long long)batch * kv_head_num;
+  const int nblocks = (n + kDecStepKeys - 1) / kDecStepKeys;
+  const int cus = device_compute_units();
+  struct Memo {
+    long long pairs;
+    int nblocks, cus, splits;
+  };
+  constexpr int kMemo = 8;
+  static thread_local Memo memo[kMemo] = {};
+  static thread_local unsigned next = 0;
+  for (const Memo &e : memo)
+    if (e.splits > 0 && e.pairs == pairs && e.nblocks == nblocks && e.cus == cus) return e.splits;
+  const int s = default_splits_model(pairs, nblocks, cus);
+  memo[next++ % kMemo] = Memo{pairs, nblocks, cus, s};
+  return s;
+}
+
+int flash_decode_effective_splits(int num_splits, int n) {
+  const int nblocks = (n + kDecStepKeys - 1) / kDecStepKeys;
+  if (num_splits > nblocks) num_splits = nblocks;  // every split holds at least one block
+  return num_splits < 1 ? 1 : num_splits;
 }
 
 size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,
@@ -501,8 +531,7 @@ size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_hea
 
 static hipError_t launch_decode_impl(DecodeParams &p, void *workspace, int batch, int kv_head_num, int num_splits,
                                      int dt, bool fused, hipStream_t stream) {
-  const int nblocks = (p.n + kDecStepKeys - 1) / kDecStepKeys;
-  p.num_splits = num_splits < nblocks ? num_splits : nblocks;  // every split holds at least one block
+  p.num_splits = flash_decode_effective_splits(num_splits, p.n);
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)kHeadDim);
   const size_t slots = (size_t)batch * kv_head_num * p.num_splits * kDecCols;
   p.ws_o = static_cast<float *>(workspace);

@@ -825,8 +825,9 @@ static hipError_t launch_prefill_t(const PrefillParams &p0, hipStream_t stream) 
   return hipGetLastError();
 }
 
-// Compute units of the current device (the kernel choice and the key-range split aim at them).
-static int device_compute_units() {
+// Compute units of the current device (the kernel choice and the split counts aim at them); 256 when
+// no device can be asked.
+int device_compute_units() {
   static std::atomic<int> cached[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;

@@ -24,11 +24,16 @@ hipError_t launch_flash_prefill(void *out, const void *q, const void *k, const v
                                 hipStream_t stream, void *workspace = nullptr);
 #endif
 
+// Compute units of the current device, cached per device; 256 when no device can be asked.
+int device_compute_units();
+
 // Split-KV decode.  rows = m * group_size <= 16 query rows per kv head.
 size_t flash_decode_workspace_bytes(int batch, int m, int group_size, int kv_head_num,
                                     int num_splits);
 int flash_decode_default_splits(int batch, int n, int kv_head_num);
 int flash_decode_max_default_splits(long long pairs);
+// The split count a launch really uses for n keys: at most one split per block of 128 keys.
+int flash_decode_effective_splits(int num_splits, int n);
 hipError_t launch_flash_decode(void *out, const void *q, const void *k, const void *v,
                                void *workspace, int batch, int m, int n, int offset,
                                int64_t kv_seq_stride, int group_size, int kv_head_num,

@@ -184,6 +184,8 @@ int llmhip_flash_decode_gqa_static(void *out, const void *q, const void *k_cache
       --num_splits;
   }
   if (num_splits > kMaxDecodeSplits) num_splits = kMaxDecodeSplits;
+  // the launch uses at most one split per 128 keys: a larger count is judged by what it becomes
+  num_splits = flash_decode_effective_splits(num_splits, n);
   // the fixed array must hold the partials of every (sequence, kv head, split)
   if (flash_decode_workspace_bytes(batch, 1, group_size, kv_head_num, num_splits) > kStaticDecodeScratchBytes)
     return LLMHIP_ERR_WORKSPACE;

@@ -21,11 +21,29 @@ def _both(ops, torch, q, k, v, batch, n, stride, g, Hkv, splits, dt):
     want, got = dev_empty(q.shape), dev_empty(q.shape)
     ops.hip_flash_decode_gqa_layer(want, dq, dk, dv, ws, wsb, batch, n, stride, g, Hkv, 128, splits, dt)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # "allocates nothing" is checked on the device itself (hipMemGetInfo), not in torch's caching allocator,
+    # which cannot see a hipMalloc made inside the library; torch's own counters must not move either
+    before_free, before_torch = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
     ops.hip_flash_decode_gqa_static_layer(got, dq, dk, dv, batch, n, stride, g, Hkv, 128, splits, dt)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == before_free and torch.cuda.memory_reserved() == before_torch
     return to_host(want), to_host(got)
+
+
+def test_device_free_bytes_see_a_library_allocation():
+    """The detector of the test above works: a device allocation made through the library (the size of the
+    per-stream scratch that the static entry point must not touch) lowers the device's free bytes, and
+    torch's counters do not notice it."""
+    import torch
+    import llm_simple_amd.ops as ops
+    torch.cuda.synchronize()
+    free0, torch0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
+    p = ctypes.c_void_p()
+    assert ops.lib.llmhip_malloc(ctypes.byref(p), 4 << 20) == 0
+    free1 = torch.cuda.mem_get_info()[0]
+    assert ops.lib.llmhip_free(p) == 0
+    assert free1 <= free0 - (4 << 20) and torch.cuda.memory_allocated() == torch0
+    assert torch.cuda.mem_get_info()[0] == free0
 
 
 @pytest.mark.parametrize("dt", [DT_BFLOAT16, DT_FLOAT16])

@@ -42,10 +42,10 @@ DT_F16 = 4
 # figures are in profiles/.  Only the shapes that were profiled have an entry.
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE summaries under profiles/ (not measured in this run)"
 MEASURED_TRAFFIC_BYTES = {
-    ("prefill", 4096): (47179 + 28672) * 1024,             # algorithmic 65536 KiB
+    ("prefill", 4096): (47165 + 28672) * 1024,             # algorithmic 65536 KiB
     ("decode", 16, 32768): (2097637 + 656) * 1024,         # algorithmic 2097152 KiB
     ("decode", 1, 32768): (131317 + 656) * 1024,           # algorithmic 131072 KiB
-    ("rope", 4096): (40753 + 36864) * 1024,                # algorithmic 75776 KiB
+    ("rope", 4096): (40753 + 36887) * 1024,                # algorithmic 75776 KiB
     ("chunked", 256, 33024): (136014 + 33556 + 33282 + 1792) * 1024,   # prefill kernel + combine
     ("chunked", 40, 131072): (537483 + 26242 + 28843 + 400) * 1024,
 }

@@ -99,12 +99,13 @@ int llmhip_flash_decode_gqa(void *out, const void *q, const void *k_cache,
 
 /* Workspace size of llmhip_flash_decode_gqa for the same (batch, group_size, kv_head_num, num_splits);
  * 0 for one split.  num_splits <= 0 gives the size that covers the default split count at any KV
- * length (at most ceil(256 / (batch * kv_head_num)) splits), so a caller that passes num_splits <= 0
+ * length (at most about one workgroup per compute unit of the device), so a caller that passes num_splits <= 0
  * to the decode call can size its workspace once. */
 size_t llmhip_flash_decode_workspace_bytes(int batch, int group_size, int kv_head_num,
                                            int head_dim, int num_splits);
 
-/* The split count the decode call uses for num_splits <= 0: about 256 workgroups in total. */
+/* The split count the decode call uses for num_splits <= 0: about one workgroup per compute unit of the
+ * current device, from a small model of the launch (whole rounds of workgroups preferred). */
 int llmhip_flash_decode_default_splits(int batch, int n, int kv_head_num);
 
 /* llmhip_flash_decode_gqa for callers that cannot allocate device memory or carry a workspace

@@ -82,6 +82,13 @@ def test_qwen_layer_through_the_device_switch_and_decode_loop_timing():
     assert 0 < t["layer_decode_us_per_step"] < 200 and 0 < t["abi_decode_us_per_step"] < 200
 
 
+def test_stream_ordered_pool_on_the_device():
+    """A block freed under queued work goes back to its own stream at once, to another stream or to host code only
+    after that work is done; the kernel that was reading it produces the right output."""
+    out = _run("op_test_pool")
+    assert "pointers as expected" in out, out
+
+
 @pytest.mark.parametrize("flags", [
     ("--m", 2048, "--n", 2048, "--k", 2048, "--dtype", "fp16"),                       # the reference CLI's defaults
     ("--m", 256, "--n", 3584, "--k", 3584, "--bias", 1, "--dtype", "bf16"),           # Qwen2.5-7B q_proj

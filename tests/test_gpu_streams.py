@@ -87,6 +87,44 @@ def test_graph_capture_and_replay():
             assert np.array_equal(a, b), f"replay {rep}"
 
 
+def test_scratch_does_not_grow_under_capture():
+    """A reference-signature call whose per-stream scratch would have to grow while its stream is being captured
+    is refused with LLMHIP_ERR_WORKSPACE (growing allocates); after the stream has been warmed up with the shape,
+    the same call is captured, and replays give the eager result."""
+    import torch
+    import llm_simple_amd.ops as ops
+    dt, H, Hkv, n = DT_BFLOAT16, 40, 8, 40000   # the default split count for this cache needs more than 4 MiB? no:
+    # 8 kv heads x 32 splits x 8320 bytes = 2.1 MB fits the first 4 MiB buffer, so ask for a chunk whose partials do not
+    m = 24                                        # 24 tokens over 40000 keys: key-range split, fp32 partials
+    need = ops.lib.llmhip_flash_attn_scratch_bytes(m, n, n - m, H // Hkv, Hkv)
+    assert need > (4 << 20), need
+    q = to_dev(normal_bits(31, (m, H, 128), dt))
+    k, v = (to_dev(normal_bits(s, (n, Hkv, 128), dt)) for s in (32, 33))
+    o, o_small = dev_empty((m, H, 128)), dev_empty((1, H, 128))
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        sp = side.cuda_stream
+        # first call on this stream: a small decode allocates the 4 MiB buffer
+        ops.hip_flash_attn_gqa_layer(o_small, q[:1], k, v, 1, 4096, 4095, H // Hkv, Hkv, 128, dt, sp)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        refused = None
+        with torch.cuda.graph(graph, stream=side):
+            cap = torch.cuda.current_stream().cuda_stream
+            ops.hip_flash_attn_gqa_layer(o_small, q[:1], k, v, 1, 4096, 4095, H // Hkv, Hkv, 128, dt, cap)   # fits: captured
+            refused = ops.lib.llmhip_flash_attn_gqa(o.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), m, n, n - m,
+                                                    H // Hkv, Hkv, 128, dt, cap)
+        assert refused == -3, refused
+    torch.cuda.synchronize()
+    # the refused call left the capture intact: the graph replays the small decode
+    want = dev_empty((1, H, 128))
+    ops.hip_flash_attn_gqa_layer(want, q[:1], k, v, 1, 4096, 4095, H // Hkv, Hkv, 128, dt)
+    o_small.fill_(0x7FFF)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(o_small), to_host(want))
+
+
 def test_measurement_aids():
     """Measurement library (libllmhip_bench.so): the clocked prefill entry returns the same output as the plain one and plausible counters; the MFMA
     ceiling probe returns a rate between a tenth of the published peak and the peak."""

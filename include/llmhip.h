@@ -189,6 +189,7 @@ int llmhip_free(void *ptr);
 int llmhip_memcpy_h2d(void *dst, const void *src, size_t bytes);
 int llmhip_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int llmhip_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *stream);
+/* Fills with a kernel (any alignment, any size), so the call may be captured into a HIP graph. */
 int llmhip_memset_async(void *dst, int value, size_t bytes, void *stream);
 int llmhip_stream_create(void **stream);
 int llmhip_stream_destroy(void *stream);

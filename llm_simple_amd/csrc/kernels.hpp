@@ -68,5 +68,7 @@ hipError_t launch_matmul_bias(void *out, const void *lhs, const void *weight, co
 void release_matmul_resources();
 hipError_t launch_add(void *out, const void *lhs, const void *rhs, size_t total, int dt,
                       hipStream_t stream);
+// dst[0 .. bytes) = (unsigned char)value with a kernel (safe to capture into a HIP graph).
+hipError_t launch_fill(void *dst, int value, size_t bytes, hipStream_t stream);
 
 }  // namespace LLMHIP_NS

@@ -300,7 +300,8 @@ int llmhip_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *stre
 }
 int llmhip_memset_async(void *dst, int value, size_t bytes, void *stream) {
   if (!dst) return LLMHIP_ERR_INVALID_ARG;
-  return from_hip(hipMemsetAsync(dst, value, bytes, as_stream(stream)));
+  // a fill kernel, not hipMemsetAsync: the call may be captured into a HIP graph
+  return from_hip(launch_fill(dst, value, bytes, as_stream(stream)));
 }
 int llmhip_stream_create(void **stream) {
   if (!stream) return LLMHIP_ERR_INVALID_ARG;

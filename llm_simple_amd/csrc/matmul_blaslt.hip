@@ -198,4 +198,31 @@ hipError_t launch_add(void *out, const void *lhs, const void *rhs, size_t total,
   return hipGetLastError();
 }
 
+// Byte fill, the kernel behind llmhip_memset_async: a memset node recorded into a HIP graph has given wrong
+// results on replays, a kernel node does not.  The bulk goes out as 16-byte stores from the first 16-byte
+// boundary on, the ragged head and tail as bytes.
+__global__ __launch_bounds__(256) void fill_kernel(unsigned char *dst, unsigned char value, size_t bytes) {
+  const size_t head = min(bytes, (size_t)((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15));
+  const size_t vecs = (bytes - head) / 16, tail0 = head + vecs * 16;
+  const uint32_t w = value * 0x01010101u;
+  const u32x4_t v = {w, w, w, w};
+  u32x4_t *mid = reinterpret_cast<u32x4_t *>(dst + head);
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < vecs; i += stride) mid[i] = v;
+  if (blockIdx.x == 0) {
+    for (size_t i = threadIdx.x; i < head; i += blockDim.x) dst[i] = value;
+    for (size_t i = tail0 + threadIdx.x; i < bytes; i += blockDim.x) dst[i] = value;
+  }
+}
+
+hipError_t launch_fill(void *dst, int value, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return hipSuccess;
+  size_t blocks = (bytes / 16 + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, static_cast<unsigned char *>(dst),
+                     (unsigned char)value, bytes);
+  return hipGetLastError();
+}
+
 }  // namespace llmhip

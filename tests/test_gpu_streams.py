@@ -125,6 +125,19 @@ def test_scratch_does_not_grow_under_capture():
     assert np.array_equal(to_host(o_small), to_host(want))
 
 
+def test_memset_async_fills_exactly_the_range():
+    """llmhip_memset_async is a fill kernel (it may be captured into a HIP graph): any alignment, any size, nothing
+    outside the range touched."""
+    import torch
+    import llm_simple_amd.ops as ops
+    for off, n in ((0, 1 << 20), (3, 1000), (5, 7), (16, 16), (1, 4097), (9, 0), (13, (1 << 22) + 11)):
+        buf = torch.full((n + 64,), 0x11, dtype=torch.uint8, device="cuda")
+        assert ops.lib.llmhip_memset_async(buf.data_ptr() + off, 0xA5, n, None) == 0
+        torch.cuda.synchronize()
+        got = buf.cpu().numpy()
+        assert (got[:off] == 0x11).all() and (got[off:off + n] == 0xA5).all() and (got[off + n:] == 0x11).all(), (off, n)
+
+
 def test_measurement_aids():
     """Measurement library (libllmhip_bench.so): the clocked prefill entry returns the same output as the plain one and plausible counters; the MFMA
     ceiling probe returns a rate between a tenth of the published peak and the peak."""

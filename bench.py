@@ -785,43 +785,47 @@ def main():
         extra["attention_block"] = r
 
     if "configs" in legs:
-        # one entry per benchmark configuration (BASELINE.json configs[0..4]); 4 and 5 summarise the legs above
-        c1 = bench_config1(ops, torch, timer, args.steps, args.warmup)
-        log(f"config 1 (Llama2-7B prefill fp16 S=256): attention {c1['us_attention']:.1f} us {c1['tflops_attention']:.0f} TFLOP/s, "
-            f"rope+append+attention {c1['us_rope_append_attention']:.1f} us, max-abs {c1['max_abs_err']:.2e} "
-            f"(layer-style {c1['max_abs_err_layer']:.2e})")
-        c2 = bench_config2(ops, torch, timer, args.steps, args.warmup)
-        log(f"config 2 (Llama2-7B decode fp16 n=512): three launches {c2['us_three_launches_cold']:.1f} us, fused step "
-            f"{c2['us_fused_step_cold']:.1f} us ({c2['gbs']:.0f} GB/s), max-abs {c2['max_abs_err']:.2e} "
-            f"(layer-style {c2['max_abs_err_layer']:.2e})")
-        torch.cuda.empty_cache()
-        c3 = bench_config3(ops, torch, timer, args.steps, args.warmup)
-        c3["decode"]["through_cpp_layer"] = layer_decode_loop()
-        lay = c3["decode"]["through_cpp_layer"]
-        log(f"config 3 (Qwen2.5-1.5B bf16): prefill 256 attention {c3['prefill']['us_attention']:.1f} us, with rope+append "
-            f"{c3['prefill']['us_rope_append_attention']:.1f} us; 256 decode steps {c3['decode']['us_total']:.0f} us = "
-            f"{c3['decode']['us_per_token']:.2f} us/token from Python; from C++: C-ABI calls "
-            f"{lay.get('abi_decode_us_per_step', float('nan')):.2f} us/token, through Qwen2AttentionLayer "
-            f"{lay.get('layer_decode_us_per_step', float('nan')):.2f} us/token (host {lay.get('layer_host_us_per_step', float('nan')):.2f}); "
-            f"max-abs prefill {c3['prefill']['max_abs_err']:.2e}, decode {c3['decode']['max_abs_err']:.2e}")
-        cfgs = [c1, c2, c3]
-        c4 = {"config": 4, "workload": "Qwen2.5-7B prefill: bf16, H=28, Hkv=4, head_dim 128, S in {1024, 4096, 8192}",
-              "dtype": "bf16", "bound": "mfma", "peak_tflops": PEAK_BF16_TFLOPS,
-              "shapes": [{"S": args.seq, "us": pre["ms_event"] * 1e3, "tflops": pre["tflops"],
-                          "frac": pre["tflops"] / PEAK_BF16_TFLOPS, "max_abs_err": pre["max_abs_err"],
-                          "max_abs_err_layer": pre["max_abs_err_layer"]}] + extra.get("prefill_other", []),
-              "frac": pre["tflops"] / PEAK_BF16_TFLOPS, "max_abs_err": pre["max_abs_err"],
-              "max_abs_err_layer": pre["max_abs_err_layer"], "max_abs_err_bar": TOL[DT_BF16]}
-        cfgs.append(c4)
-        if "decode_all" in extra:
-            c5 = {"config": 5, "workload": "Qwen2.5-32B decode: bf16, H=40, Hkv=8, head_dim 128, n in {4096, 16384, 32768}, "
-                                           "batch in {1, 16}, cold", "dtype": "bf16", "bound": "hbm", "peak_gbs": PEAK_HBM_GBS,
-                  "shapes": extra["decode_all"], "frac": extra["roofline_decode"]["frac"],
-                  "max_abs_err": max(x["max_abs_err"] for x in extra["decode_all"]),
-                  "max_abs_err_layer": max(x["max_abs_err_layer"] for x in extra["decode_all"]),
-                  "max_abs_err_bar": TOL[DT_BF16]}
-            cfgs.append(c5)
-        extra["configs"] = cfgs
+        try:
+            # one entry per benchmark configuration (BASELINE.json configs[0..4]); 4 and 5 summarise the legs above
+            c1 = bench_config1(ops, torch, timer, args.steps, args.warmup)
+            log(f"config 1 (Llama2-7B prefill fp16 S=256): attention {c1['us_attention']:.1f} us {c1['tflops_attention']:.0f} TFLOP/s, "
+                f"rope+append+attention {c1['us_rope_append_attention']:.1f} us, max-abs {c1['max_abs_err']:.2e} "
+                f"(layer-style {c1['max_abs_err_layer']:.2e})")
+            c2 = bench_config2(ops, torch, timer, args.steps, args.warmup)
+            log(f"config 2 (Llama2-7B decode fp16 n=512): three launches {c2['us_three_launches_cold']:.1f} us, fused step "
+                f"{c2['us_fused_step_cold']:.1f} us ({c2['gbs']:.0f} GB/s), max-abs {c2['max_abs_err']:.2e} "
+                f"(layer-style {c2['max_abs_err_layer']:.2e})")
+            torch.cuda.empty_cache()
+            c3 = bench_config3(ops, torch, timer, args.steps, args.warmup)
+            c3["decode"]["through_cpp_layer"] = layer_decode_loop()
+            lay = c3["decode"]["through_cpp_layer"]
+            log(f"config 3 (Qwen2.5-1.5B bf16): prefill 256 attention {c3['prefill']['us_attention']:.1f} us, with rope+append "
+                f"{c3['prefill']['us_rope_append_attention']:.1f} us; 256 decode steps {c3['decode']['us_total']:.0f} us = "
+                f"{c3['decode']['us_per_token']:.2f} us/token from Python; from C++: C-ABI calls "
+                f"{lay.get('abi_decode_us_per_step', float('nan')):.2f} us/token, through Qwen2AttentionLayer "
+                f"{lay.get('layer_decode_us_per_step', float('nan')):.2f} us/token (host {lay.get('layer_host_us_per_step', float('nan')):.2f}); "
+                f"max-abs prefill {c3['prefill']['max_abs_err']:.2e}, decode {c3['decode']['max_abs_err']:.2e}")
+            cfgs = [c1, c2, c3]
+            c4 = {"config": 4, "workload": "Qwen2.5-7B prefill: bf16, H=28, Hkv=4, head_dim 128, S in {1024, 4096, 8192}",
+                  "dtype": "bf16", "bound": "mfma", "peak_tflops": PEAK_BF16_TFLOPS,
+                  "shapes": [{"S": args.seq, "us": pre["ms_event"] * 1e3, "tflops": pre["tflops"],
+                              "frac": pre["tflops"] / PEAK_BF16_TFLOPS, "max_abs_err": pre["max_abs_err"],
+                              "max_abs_err_layer": pre["max_abs_err_layer"]}] + extra.get("prefill_other", []),
+                  "frac": pre["tflops"] / PEAK_BF16_TFLOPS, "max_abs_err": pre["max_abs_err"],
+                  "max_abs_err_layer": pre["max_abs_err_layer"], "max_abs_err_bar": TOL[DT_BF16]}
+            cfgs.append(c4)
+            if "decode_all" in extra:
+                c5 = {"config": 5, "workload": "Qwen2.5-32B decode: bf16, H=40, Hkv=8, head_dim 128, n in {4096, 16384, 32768}, "
+                                               "batch in {1, 16}, cold", "dtype": "bf16", "bound": "hbm", "peak_gbs": PEAK_HBM_GBS,
+                      "shapes": extra["decode_all"], "frac": extra["roofline_decode"]["frac"],
+                      "max_abs_err": max(x["max_abs_err"] for x in extra["decode_all"]),
+                      "max_abs_err_layer": max(x["max_abs_err_layer"] for x in extra["decode_all"]),
+                      "max_abs_err_bar": TOL[DT_BF16]}
+                cfgs.append(c5)
+            extra["configs"] = cfgs
+        except Exception as e:  # the headline line must still be printed
+            log(f"configs leg failed: {e!r}")
+            extra["configs_error"] = repr(e)
 
     if args.calib_copy:
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()
